@@ -921,6 +921,144 @@ std::function<void(A...)> checked(const char* name, void (*f)(A...)) {
   };
 }
 
+
+// ------------------------------------------------------------------ post-norm fp32 residual / sigmoid attention
+// activations are bf16 or fp32 (one type per call); residual, norm weights and state are fp32
+bool act_f32(const Tensor& t) {
+  CHECK_DEV(t);
+  TORCH_CHECK(t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat, "activations must be bfloat16 or float32");
+  return t.scalar_type() == at::kFloat;
+}
+#define CHECK_F32(x) \
+  CHECK_DEV(x);      \
+  CHECK_DT(x, at::kFloat); \
+  CHECK_CONTIG(x)
+#define CHECK_I32(x) \
+  CHECK_DEV(x);      \
+  CHECK_DT(x, at::kInt); \
+  CHECK_CONTIG(x)
+
+void embed_pos(Tensor x, Tensor ids, Tensor pos, Tensor embed, Tensor ptab) {
+  CHECK_F32(x); CHECK_I32(ids); CHECK_I32(pos);
+  const bool f32 = act_f32(embed);
+  TORCH_CHECK(ptab.scalar_type() == embed.scalar_type() && ptab.is_cuda());
+  CHECK_CONTIG(embed); CHECK_CONTIG(ptab);
+  TORCH_CHECK(x.dim() == 2 && embed.dim() == 2 && ptab.dim() == 2);
+  const int H = (int)x.size(1);
+  TORCH_CHECK(embed.size(1) == H && ptab.size(1) == H && ids.numel() == x.size(0) && pos.numel() == x.size(0));
+  nga::launch_embed_pos(x.data_ptr<float>(), ids.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), embed.data_ptr(),
+                        ptab.data_ptr(), x.size(0), H, (int)embed.size(0), (int)ptab.size(0), f32, cur_stream(x));
+}
+
+void rmsnorm_residual(Tensor x, Tensor y, Tensor w, double eps, c10::optional<Tensor> cast_out) {
+  CHECK_F32(x); CHECK_F32(w);
+  const bool f32 = act_f32(y);
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && y.size(0) == x.size(0) && y.size(1) == x.size(1) && y.stride(1) == 1);
+  TORCH_CHECK(w.numel() == x.size(1));
+  void* co = nullptr;
+  if (cast_out.has_value()) {
+    TORCH_CHECK(cast_out->is_cuda() && cast_out->scalar_type() == y.scalar_type() && cast_out->is_contiguous() &&
+                cast_out->sizes() == x.sizes());
+    co = cast_out->data_ptr();
+  }
+  nga::launch_rmsnorm_residual(x.data_ptr<float>(), y.data_ptr(), y.stride(0), w.data_ptr<float>(), (float)eps,
+                               x.size(0), (int)x.size(1), co, f32, cur_stream(x));
+}
+
+void rmsnorm_f32(Tensor out, Tensor x, c10::optional<Tensor> rows, Tensor w, double eps) {
+  CHECK_F32(x); CHECK_F32(w); CHECK_CONTIG(out);
+  const bool f32 = act_f32(out);
+  TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && out.size(1) == x.size(1) && w.numel() == x.size(1));
+  const int64_t* rp = nullptr;
+  if (rows.has_value()) {
+    CHECK_DEV(*rows); CHECK_DT(*rows, at::kLong); CHECK_CONTIG(*rows);
+    TORCH_CHECK(rows->numel() == out.size(0));
+    rp = rows->data_ptr<int64_t>();
+  } else {
+    TORCH_CHECK(out.size(0) == x.size(0));
+  }
+  nga::launch_rmsnorm_f32(out.data_ptr(), x.data_ptr<float>(), rp, w.data_ptr<float>(), (float)eps, out.size(0),
+                          (int)x.size(1), f32, cur_stream(x));
+}
+
+void token_shift(Tensor h, Tensor x, Tensor mu, Tensor src, Tensor state) {
+  CHECK_F32(x); CHECK_F32(mu); CHECK_F32(state); CHECK_I32(src); CHECK_CONTIG(h);
+  const bool f32 = act_f32(h);
+  TORCH_CHECK(x.dim() == 2 && h.sizes() == x.sizes() && mu.numel() == x.size(1) && src.numel() == x.size(0));
+  TORCH_CHECK(state.dim() == 2 && state.size(1) == x.size(1));
+  nga::launch_token_shift(h.data_ptr(), x.data_ptr<float>(), mu.data_ptr<float>(), src.data_ptr<int32_t>(),
+                          state.data_ptr<float>(), x.size(0), (int)x.size(1), f32, cur_stream(x));
+}
+
+void shift_save(Tensor state, Tensor x, Tensor last_row, Tensor slot) {
+  CHECK_F32(state); CHECK_F32(x); CHECK_I32(last_row); CHECK_I32(slot);
+  TORCH_CHECK(state.dim() == 2 && x.dim() == 2 && state.size(1) == x.size(1) && last_row.numel() == slot.numel());
+  nga::launch_shift_save(state.data_ptr<float>(), x.data_ptr<float>(), last_row.data_ptr<int32_t>(),
+                         slot.data_ptr<int32_t>(), (int)slot.numel(), (int)x.size(1), cur_stream(x));
+}
+
+void glu_gelu_tanh(Tensor out, Tensor x) {
+  const bool f32 = act_f32(x);
+  CHECK_CONTIG(out); CHECK_CONTIG(x);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == x.scalar_type());
+  TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && x.size(1) == 2 * out.size(1) && x.size(0) == out.size(0));
+  nga::launch_glu_gelu_tanh(out.data_ptr(), x.data_ptr(), x.size(0), (int)out.size(1), f32, cur_stream(x));
+}
+
+// K [blocks, Hkv, 64, dk] and V^T [blocks, Hkv, dv, 64] pages of the activation type
+void check_sig_pages(const Tensor& proj, const Tensor& kc, const Tensor& vc, int64_t Hkv, int64_t dk, int64_t dv) {
+  TORCH_CHECK(kc.is_cuda() && vc.is_cuda() && kc.is_contiguous() && vc.is_contiguous());
+  TORCH_CHECK(kc.scalar_type() == proj.scalar_type() && vc.scalar_type() == proj.scalar_type(),
+              "KV pages must have the activation type");
+  TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.size(0) == vc.size(0) && kc.size(1) == Hkv && vc.size(1) == Hkv &&
+                  kc.size(2) == 64 && kc.size(3) == dk && vc.size(2) == dv && vc.size(3) == 64,
+              "KV pages must be K [blocks, Hkv, 64, dk] and V^T [blocks, Hkv, dv, 64]");
+}
+
+void qk_norm_cache(Tensor proj, Tensor qw, Tensor kw, double eps, Tensor slots, Tensor kc, Tensor vc, int64_t Hq,
+                   int64_t Hkv, int64_t dk, int64_t dv) {
+  const bool f32 = act_f32(proj);
+  CHECK_F32(qw); CHECK_F32(kw); CHECK_I32(slots);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(1) >= (Hq + Hkv) * dk + Hkv * dv);
+  TORCH_CHECK(qw.numel() == Hq * dk && kw.numel() == Hkv * dk && slots.numel() == proj.size(0));
+  TORCH_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && dk > 0 && dv > 0);
+  check_sig_pages(proj, kc, vc, Hkv, dk, dv);
+  nga::launch_qk_norm_cache(proj.data_ptr(), proj.stride(0), qw.data_ptr<float>(), kw.data_ptr<float>(), (float)eps,
+                            slots.data_ptr<int32_t>(), kc.data_ptr(), vc.data_ptr(), proj.size(0), (int)Hq, (int)Hkv,
+                            (int)dk, (int)dv, f32, cur_stream(proj));
+}
+
+void sigmoid_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc, Tensor block_tables,
+                       Tensor tok_seq, Tensor pos, int64_t Hq, int64_t Hkv, int64_t dk, int64_t dv, double scale,
+                       int64_t window, int64_t keep_first, Tensor r1, Tensor r2, Tensor pb) {
+  const bool f32 = act_f32(q);
+  CHECK_F32(r1); CHECK_F32(r2); CHECK_F32(pb); CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
+  CHECK_CONTIG(out);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == q.scalar_type());
+  const int64_t T = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == Hq * dk, "q must be [T, Hq * dk] rows");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == Hq * dv);
+  TORCH_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && dk > 0 && dk <= 1024 && dv > 0 && dv <= 256,
+              "sigmoid_attention: dk <= 1024, dv <= 256");
+  TORCH_CHECK(window > 0 && keep_first >= 0);
+  TORCH_CHECK(r1.numel() == Hq && r2.numel() == Hq && pb.numel() == Hq);
+  TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);
+  check_sig_pages(q, kc, vc, Hkv, dk, dv);
+  const void* gp = nullptr;
+  int64_t gs = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == q.scalar_type() && gate->dim() == 2 && gate->size(0) == T &&
+                gate->size(1) == Hq * dv && gate->stride(1) == 1);
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
+  }
+  nga::launch_sigmoid_attention(out.data_ptr(), q.data_ptr(), q.stride(0), gp, gs, kc.data_ptr(), vc.data_ptr(),
+                                block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
+                                tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T, (int)Hq, (int)Hkv, (int)dk,
+                                (int)dv, (float)scale, (int)window, (int)keep_first, r1.data_ptr<float>(),
+                                r2.data_ptr<float>(), pb.data_ptr<float>(), f32, cur_stream(q));
+}
+
 }  // namespace
 
 
@@ -974,6 +1112,14 @@ PYBIND11_MODULE(_C, m) {
   m.def("layernorm", checked("layernorm", &layernorm));
   m.def("add_layernorm", checked("add_layernorm", &add_layernorm));
   m.def("gelu_tanh_mul", checked("gelu_tanh_mul", &gelu_tanh_mul));
+  m.def("embed_pos", checked("embed_pos", &embed_pos));
+  m.def("rmsnorm_residual", checked("rmsnorm_residual", &rmsnorm_residual));
+  m.def("rmsnorm_f32", checked("rmsnorm_f32", &rmsnorm_f32));
+  m.def("token_shift", checked("token_shift", &token_shift));
+  m.def("shift_save", checked("shift_save", &shift_save));
+  m.def("glu_gelu_tanh", checked("glu_gelu_tanh", &glu_gelu_tanh));
+  m.def("qk_norm_cache", checked("qk_norm_cache", &qk_norm_cache));
+  m.def("sigmoid_attention", checked("sigmoid_attention", &sigmoid_attention));
   m.def("silu_mul", checked("silu_mul", &silu_mul));
   m.def("bias_gelu", checked("bias_gelu", &bias_gelu));
   m.def("rope_cache", checked("rope_cache", &rope_cache));

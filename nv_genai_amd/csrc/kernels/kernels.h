@@ -223,4 +223,27 @@ void launch_splitk_reduce(const float* P, int S, int M, int N, uint16_t* out, in
 void launch_splitk_add_rmsnorm(const float* P, int S, int M, uint16_t* resid, const uint16_t* w,
                                float eps, int H, uint16_t* out, hipStream_t stream);
 
+// postnorm.hip: fp32 residual stream rows (f32: activations / tables are float, else bf16)
+void launch_embed_pos(float* x, const int32_t* ids, const int32_t* pos, const void* embed, const void* ptab,
+                      int64_t T, int H, int vocab, int max_pos, bool f32, hipStream_t stream);
+void launch_rmsnorm_residual(float* x, const void* y, int64_t y_stride, const float* w, float eps, int64_t T, int H,
+                             void* cast_out, bool f32, hipStream_t stream);
+void launch_rmsnorm_f32(void* out, const float* x, const int64_t* rows, const float* w, float eps, int64_t T, int H,
+                        bool f32, hipStream_t stream);
+void launch_token_shift(void* h, const float* x, const float* mu, const int32_t* src, const float* state, int64_t T,
+                        int H, bool f32, hipStream_t stream);
+void launch_shift_save(float* state, const float* x, const int32_t* last_row, const int32_t* slot, int n, int H,
+                       hipStream_t stream);
+void launch_glu_gelu_tanh(void* out, const void* in, int64_t T, int F, bool f32, hipStream_t stream);
+
+// sigmoid_attention.hip: K [blocks, Hkv, 64, dk], V^T [blocks, Hkv, dv, 64] pages, bf16 or fp32
+void launch_qk_norm_cache(void* proj, int64_t stride, const float* qw, const float* kw, float eps,
+                          const int32_t* slots, void* kc, void* vc, int64_t T, int Hq, int Hkv, int dk, int dv,
+                          bool f32, hipStream_t stream);
+void launch_sigmoid_attention(void* out, const void* q, int64_t q_stride, const void* gate, int64_t g_stride,
+                              const void* kc, const void* vc, const int32_t* block_tables, int max_blocks,
+                              const int32_t* tok_seq, const int32_t* pos, int64_t T, int Hq, int Hkv, int dk, int dv,
+                              float scale, int window, int keep_first, const float* r1, const float* r2,
+                              const float* pb, bool f32, hipStream_t stream);
+
 }  // namespace nga

@@ -1,0 +1,171 @@
+// Row kernels of post-norm decoders with an fp32 residual stream and a token-shift state:
+//
+//   embed_pos         x[t]  = embed[id[t]] + pos_table[pos[t]]                    (fp32 out)
+//   rmsnorm_residual  x[t] += y[t] * rsqrt(mean(y[t]^2) + eps) * w  (+ a cast copy of x[t])
+//   token_shift       h[t]  = x[t] + (prev(t) - x[t]) * mu, prev(t) the same layer's input one
+//                     token earlier: a row of this step, a state slot, or zeros (position 0)
+//   shift_save        state[slot[i]] = x[last_row[i]] for every sequence of the step
+//   glu_gelu_tanh     [T, 2F] = [gate | up] -> gelu_tanh(gate) * up, any F, bf16 or fp32
+//
+// The residual, the norms and the shift interpolation are fp32 whatever the activation type T
+// (bf16 storage as uint16_t, or float). Memory-bound: one workgroup per row, columns strided
+// over the lanes (no alignment assumed: widths need not be multiples of 8).
+#include "common.h"
+#include "kernels.h"
+
+namespace nga {
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+template <typename T>
+__global__ void __launch_bounds__(256) embed_pos_kernel(float* __restrict__ x, const int32_t* __restrict__ ids,
+                                                        const int32_t* __restrict__ pos, const T* __restrict__ embed,
+                                                        const T* __restrict__ ptab, int H, int vocab, int max_pos) {
+  const int64_t row = blockIdx.x;
+  int id = ids[row], p = pos[row];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // padding rows of a captured step
+  p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+  for (int c = threadIdx.x; c < H; c += blockDim.x)
+    x[row * H + c] = ldf(embed + (int64_t)id * H + c) + ldf(ptab + (int64_t)p * H + c);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) rmsnorm_residual_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                                               int64_t y_stride, const float* __restrict__ w,
+                                                               float eps, int H, T* __restrict__ cast_out) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float v = ldf(yr + c);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float v = x[row * H + c] + ldf(yr + c) * r * w[c];
+    x[row * H + c] = v;
+    if (cast_out) stf(cast_out + row * H + c, v);
+  }
+}
+
+// out = rmsnorm(x) * w of fp32 rows (the model's last norm), written in T
+template <typename T>
+__global__ void __launch_bounds__(256) rmsnorm_f32_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                          const int64_t* __restrict__ rows, const float* __restrict__ w,
+                                                          float eps, int H) {
+  __shared__ float red[4];
+  const int64_t src = rows ? rows[blockIdx.x] : (int64_t)blockIdx.x;
+  const float* xr = x + src * H;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) ss += xr[c] * xr[c];
+  ss = block_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += blockDim.x) stf(out + (int64_t)blockIdx.x * H + c, xr[c] * r * w[c]);
+}
+
+// src[t] >= 0: row of x; -1: zeros; <= -2: state slot -(src + 2)
+template <typename T>
+__global__ void __launch_bounds__(256) token_shift_kernel(T* __restrict__ h, const float* __restrict__ x,
+                                                          const float* __restrict__ mu, const int32_t* __restrict__ src,
+                                                          const float* __restrict__ state, int H) {
+  const int64_t row = blockIdx.x;
+  const int s = src[row];
+  const float* prev = s >= 0 ? x + (int64_t)s * H : (s == -1 ? nullptr : state + (int64_t)(-(s + 2)) * H);
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float v = x[row * H + c];
+    const float p = prev ? prev[c] : 0.f;
+    stf(h + row * H + c, v + (p - v) * mu[c]);
+  }
+}
+
+__global__ void __launch_bounds__(256) shift_save_kernel(float* __restrict__ state, const float* __restrict__ x,
+                                                         const int32_t* __restrict__ last_row,
+                                                         const int32_t* __restrict__ slot, int H) {
+  const int s = slot[blockIdx.x], r = last_row[blockIdx.x];
+  if (s < 0 || r < 0) return;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) state[(int64_t)s * H + c] = x[(int64_t)r * H + c];
+}
+
+__device__ __forceinline__ float gelu_tanh_exact(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) glu_gelu_tanh_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                                            int64_t T_rows, int F) {
+  const int64_t total = T_rows * F;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / F;
+    const int c = (int)(i - t * F);
+    stf(out + i, gelu_tanh_exact(ldf(in + t * 2 * F + c)) * ldf(in + t * 2 * F + F + c));
+  }
+}
+
+}  // namespace
+
+void launch_embed_pos(float* x, const int32_t* ids, const int32_t* pos, const void* embed, const void* ptab,
+                      int64_t T, int H, int vocab, int max_pos, bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    embed_pos_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(x, ids, pos, (const float*)embed,
+                                                                  (const float*)ptab, H, vocab, max_pos);
+  else
+    embed_pos_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>(x, ids, pos, (const uint16_t*)embed,
+                                                                     (const uint16_t*)ptab, H, vocab, max_pos);
+}
+
+void launch_rmsnorm_residual(float* x, const void* y, int64_t y_stride, const float* w, float eps, int64_t T, int H,
+                             void* cast_out, bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    rmsnorm_residual_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const float*)y, y_stride, w, eps, H,
+                                                                         (float*)cast_out);
+  else
+    rmsnorm_residual_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const uint16_t*)y, y_stride, w, eps,
+                                                                            H, (uint16_t*)cast_out);
+}
+
+void launch_rmsnorm_f32(void* out, const float* x, const int64_t* rows, const float* w, float eps, int64_t T, int H,
+                        bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    rmsnorm_f32_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>((float*)out, x, rows, w, eps, H);
+  else
+    rmsnorm_f32_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)out, x, rows, w, eps, H);
+}
+
+void launch_token_shift(void* h, const float* x, const float* mu, const int32_t* src, const float* state, int64_t T,
+                        int H, bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    token_shift_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>((float*)h, x, mu, src, state, H);
+  else
+    token_shift_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)h, x, mu, src, state, H);
+}
+
+void launch_shift_save(float* state, const float* x, const int32_t* last_row, const int32_t* slot, int n, int H,
+                       hipStream_t stream) {
+  if (n == 0) return;
+  shift_save_kernel<<<dim3((unsigned)n), 256, 0, stream>>>(state, x, last_row, slot, H);
+}
+
+void launch_glu_gelu_tanh(void* out, const void* in, int64_t T, int F, bool f32, hipStream_t stream) {
+  if (T == 0 || F == 0) return;
+  int64_t g = (T * F + 255) / 256;
+  if (g > 8192) g = 8192;
+  if (f32)
+    glu_gelu_tanh_kernel<float><<<dim3((unsigned)g), 256, 0, stream>>>((float*)out, (const float*)in, T, F);
+  else
+    glu_gelu_tanh_kernel<uint16_t><<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, T, F);
+}
+
+}  // namespace nga

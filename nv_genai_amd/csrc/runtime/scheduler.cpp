@@ -135,6 +135,7 @@ struct Seq {
   int64_t arrival;
   int preemptions = 0;
   int64_t enq_step = 0;  // scheduler step at which it (re)entered the waiting queue
+  int slot = -1;         // state slot (models with per-sequence recurrent state), -1: none
 };
 
 class Scheduler {
@@ -177,6 +178,92 @@ class Scheduler {
     mixed_wait_ = std::max(0, max_wait_steps);
   }
   int last_num_decode() const { return last_nd_; }
+
+  // State slots: a model that carries per-sequence state besides the paged KV (a token-shift
+  // row, a recurrent state) keeps it in one of `n` fixed slots. A sequence holds a slot from
+  // admission until it finishes or is preempted (its state is recomputed with its KV).
+  void set_state_slots(int n) {
+    if (!running_.empty()) throw std::runtime_error("set_state_slots with running sequences");
+    free_slots_.clear();
+    for (int i = n - 1; i >= 0; --i) free_slots_.push_back(i);
+    slots_on_ = n > 0;
+  }
+  int free_state_slots() const { return (int)free_slots_.size(); }
+  int state_slot(int64_t id) const { return seqs_.at(id).slot; }
+  // slot of each row's sequence (rows of the last schedule: seq_ids[0..n))
+  void state_slots(py::array_t<int64_t> seq_ids, int n, py::array_t<int32_t> out) const {
+    auto a = seq_ids.unchecked<1>();
+    auto o = out.mutable_unchecked<1>();
+    for (int i = 0; i < n; ++i) o(i) = seqs_.at(a(i)).slot;
+  }
+
+  // More tokens of a sequence whose prompt arrives in portions (replay of a recorded schedule).
+  void extend(int64_t id, const std::vector<int32_t>& toks) {
+    Seq& s = seqs_.at(id);
+    if ((int)(s.toks.size() + toks.size()) > max_len_) throw std::runtime_error("sequence exceeds max_model_len");
+    s.toks.insert(s.toks.end(), toks.begin(), toks.end());
+    s.prompt_len = (int)s.toks.size();
+  }
+
+  // Replay: lay out exactly these rows, `counts[i]` next tokens of sequence `ids[i]`, instead
+  // of choosing them. A waiting sequence is admitted (no prefix-cache lookup: the caller
+  // fixes what is computed), pages are allocated as the rows need them; rows that continue a
+  // sequence by one token come first (the decode rows of a mixed step), in the given order.
+  // Returns (kind, rows, tokens) like schedule(); throws when the pool or the slots run out.
+  py::tuple schedule_rows(const std::vector<int64_t>& ids, const std::vector<int>& counts,
+                          py::array_t<int32_t> input_ids, py::array_t<int32_t> positions,
+                          py::array_t<int32_t> slots, py::array_t<int32_t> cu_q, py::array_t<int32_t> ctx,
+                          py::array_t<int32_t> block_tables, py::array_t<int64_t> seq_ids,
+                          py::array_t<int32_t> sample) {
+    Bufs B{input_ids.mutable_unchecked<1>(), positions.mutable_unchecked<1>(),
+           slots.mutable_unchecked<1>(), cu_q.mutable_unchecked<1>(), ctx.mutable_unchecked<1>(),
+           block_tables.mutable_unchecked<2>(), seq_ids.mutable_unchecked<1>(),
+           sample.mutable_unchecked<1>()};
+    if (ids.size() != counts.size()) throw std::runtime_error("schedule_rows: ids and counts differ in length");
+    if ((int)ids.size() > std::min<int>((int)B.sid.shape(0), max_seqs_))
+      throw std::runtime_error("schedule_rows: more rows than max_num_seqs");
+    ++step_;
+    last_nd_ = 0;
+    std::vector<int64_t> dec, pre;
+    std::vector<int> pre_n;
+    int total = 0;
+    for (size_t i = 0; i < ids.size(); ++i) {
+      Seq& s = seqs_.at(ids[i]);
+      const int n = counts[i];
+      if (n <= 0 || s.computed + n > (int)s.toks.size())
+        throw std::runtime_error("schedule_rows: row outside the sequence's tokens");
+      if (std::count(ids.begin(), ids.end(), ids[i]) != 1) throw std::runtime_error("schedule_rows: duplicate row");
+      total += n;
+      if (s.status == WAITING) {
+        if ((int)running_.size() >= max_seqs_) throw std::runtime_error("schedule_rows: max_num_seqs running");
+        take_slot(s);
+        waiting_.erase(std::find(waiting_.begin(), waiting_.end(), s.id));
+        running_.push_back(s.id);
+        s.status = RUNNING;
+      }
+      while ((int)s.blocks.size() * bs_ < s.computed + n) {
+        const int b = bm_.alloc();
+        if (b < 0) throw std::runtime_error("schedule_rows: KV pool exhausted");
+        s.blocks.push_back(b);
+      }
+      if (n == 1 && s.computed > 0) {
+        dec.push_back(s.id);
+      } else {
+        pre.push_back(s.id);
+        pre_n.push_back(n);
+      }
+    }
+    if (total > std::min<int>((int)B.ids.shape(0), max_tokens_))
+      throw std::runtime_error("schedule_rows: more tokens than max_batched_tokens");
+    if (ids.empty()) return py::make_tuple(0, 0, 0);
+    const std::vector<int> ones(dec.size(), 1);
+    B.cq(0) = 0;
+    int t = fill_rows(B, dec, ones, 0, 0);
+    if (pre.empty()) return py::make_tuple(2, (int)dec.size(), t);
+    last_nd_ = (int)dec.size();
+    t = fill_rows(B, pre, pre_n, (int)dec.size(), t);
+    return py::make_tuple(dec.empty() ? 1 : 3, (int)(dec.size() + pre.size()), t);
+  }
 
   // Fill the step buffers. Returns (kind, num_seqs, num_tokens); kind 0 idle, 1 prefill,
   // 2 decode, 3 mixed (rows [0, last_num_decode()) decode one token each, the rest prefill).
@@ -293,6 +380,7 @@ class Scheduler {
   // queue and recomputes (prefix-cached blocks still hit), like a preempted sequence.
   py::tuple fork(int64_t pid, int64_t cid) {
     if (seqs_.count(cid)) throw std::runtime_error("duplicate sequence id");
+    if (slots_on_) throw std::runtime_error("fork of a sequence with a state slot is not supported");
     const Seq& p = seqs_.at(pid);
     Seq c;
     c.id = cid;
@@ -338,6 +426,7 @@ class Scheduler {
     Seq& s = it->second;
     for (int b : s.blocks) bm_.release(b);
     s.blocks.clear();
+    drop_slot(s);
     if (s.status == RUNNING)
       running_.erase(std::find(running_.begin(), running_.end(), id));
     else if (s.status == WAITING) {
@@ -390,6 +479,7 @@ class Scheduler {
       const int64_t id = waiting_.front();
       Seq& s = seqs_.at(id);
       if (!admit(s)) break;
+      take_slot(s);
       waiting_.pop_front();
       running_.push_back(id);
       s.status = RUNNING;
@@ -537,7 +627,19 @@ class Scheduler {
     return t;
   }
 
+  void take_slot(Seq& s) {
+    if (!slots_on_ || s.slot >= 0) return;
+    if (free_slots_.empty()) throw std::runtime_error("no free state slot");
+    s.slot = free_slots_.back();
+    free_slots_.pop_back();
+  }
+  void drop_slot(Seq& s) {
+    if (s.slot >= 0) free_slots_.push_back(s.slot);
+    s.slot = -1;
+  }
+
   bool admit(Seq& s) {
+    if (slots_on_ && free_slots_.empty()) return false;
     // prefix-cache lookup over full blocks, keeping >= 1 token to compute
     const int n = (int)s.toks.size();
     std::vector<int32_t> got;
@@ -585,6 +687,7 @@ class Scheduler {
     for (int b : s.blocks) bm_.release(b);
     s.blocks.clear();
     s.hashes.clear();
+    drop_slot(s);
     s.computed = 0;
     s.status = WAITING;
     s.preemptions += 1;
@@ -614,6 +717,8 @@ class Scheduler {
   int64_t step_ = 0;
   int align_ = 1;
   int last_nd_ = 0;
+  bool slots_on_ = false;
+  std::vector<int> free_slots_;
 };
 
 }  // namespace
@@ -669,7 +774,13 @@ PYBIND11_MODULE(_rt, m) {
       .def("set_mixed_prefill_tokens", &Scheduler::set_mixed_prefill_tokens)
       .def("set_token_alignment", &Scheduler::set_token_alignment)
       .def("set_mixed_min_tokens", &Scheduler::set_mixed_min_tokens)
-      .def("last_num_decode", &Scheduler::last_num_decode);
+      .def("last_num_decode", &Scheduler::last_num_decode)
+      .def("set_state_slots", &Scheduler::set_state_slots)
+      .def("free_state_slots", &Scheduler::free_state_slots)
+      .def("state_slot", &Scheduler::state_slot)
+      .def("state_slots", &Scheduler::state_slots)
+      .def("extend", &Scheduler::extend)
+      .def("schedule_rows", &Scheduler::schedule_rows);
   register_bm25(m);
   register_text(m);
   register_json(m);

@@ -34,7 +34,8 @@ import torch
 from .. import ops
 from ..observability.markers import gpu_range
 from .._native import rt
-from ..models.config import LlamaConfig, llama_config
+from ..models.config import LLAMA_PRESETS, LlamaConfig, llama_config
+from ..models.registry import is_model_dir, load_model
 from ..models.llama import AttnMeta, LlamaModel
 from ..parallel.dist import ParallelContext, get_context
 from ..utils.faults import FaultInjector
@@ -150,6 +151,7 @@ class EngineConfig:
     # numerics checks: every step's fp32 logits of its sampling rows are copied (before
     # sampling, inside captured graphs too) to ``LLMEngine.d_tap`` for ``step_hook``
     logits_tap: bool = False
+    dtype: str = "bfloat16"   # model dtype: bfloat16, or float32 (true fp32 everywhere: numerics checks)
 
 
 _INERT = Request(id=-1, prompt_ids=[0], params=SamplingParams(temperature=0.0))
@@ -166,9 +168,22 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
             device = str(self.p.device) if self.p.device.type == "cuda" else (
                 "cuda" if torch.cuda.is_available() else "cpu")
         self.device = torch.device(device)
+        mdtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[cfg.dtype]
+        if model is None and model_cfg is None and is_model_dir(cfg.model):
+            # a model folder: config.json picks the class (models/registry.py)
+            model = load_model(cfg.model, self.device, mdtype, pctx=self.p)
+        if model is not None and model_cfg is None and not (isinstance(cfg.model, str) and cfg.model in LLAMA_PRESETS):
+            model_cfg = model.cfg
         self.mcfg = model_cfg or llama_config(cfg.model, max_position=max(cfg.max_model_len, 256))
-        self.model = model or LlamaModel(self.mcfg, self.device, pctx=self.p, seed=cfg.seed,
+        if model is None and not isinstance(self.mcfg, LlamaConfig):
+            from ..models.registry import model_class_for
+
+            model = model_class_for(self.mcfg)(self.mcfg, self.device, dtype=mdtype, pctx=self.p, seed=cfg.seed,
+                                               weights=weights)
+        self.model = model or LlamaModel(self.mcfg, self.device, dtype=mdtype, pctx=self.p, seed=cfg.seed,
                                          weights=weights, fp8=cfg.fp8)
+        if cfg.max_model_len > getattr(self.mcfg, "max_position", cfg.max_model_len) and not isinstance(self.mcfg, LlamaConfig):
+            raise ValueError(f"max_model_len {cfg.max_model_len} exceeds the model's {self.mcfg.max_position} positions")
         if cfg.fp8 and not self.model.fp8:
             self.model.quantize_fp8()
         self.model.sequence_parallel = cfg.sequence_parallel
@@ -192,9 +207,15 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         self.num_blocks = int(nb)
         self.model.allocate_kv_cache(self.num_blocks, cfg.block_size, cfg.kv_cache_dtype, cfg.kv_scales)
         self.max_blocks = (cfg.max_model_len + cfg.block_size - 1) // cfg.block_size
+        # per-sequence state besides the KV pages (token shift, recurrent layers): one slot per
+        # running sequence, handed out by the scheduler; cached prefix pages carry no such state
+        self.stateful = bool(getattr(self.model, "stateful", False))
         self.sched = rt.Scheduler(self.num_blocks, cfg.block_size, cfg.max_num_seqs,
                                   cfg.max_batched_tokens, cfg.max_model_len,
-                                  cfg.enable_prefix_caching)
+                                  cfg.enable_prefix_caching and getattr(self.model, "supports_prefix_cache", True))
+        if self.stateful:
+            self.sched.set_state_slots(cfg.max_num_seqs)
+            self.model.allocate_state(cfg.max_num_seqs)
         self.sched.set_mixed_prefill_tokens(cfg.mixed_prefill_tokens)
         self.sched.set_token_alignment(cfg.token_alignment)
         self.sched.set_mixed_min_tokens(cfg.mixed_min_tokens, cfg.mixed_max_wait)
@@ -216,6 +237,9 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         self.h_seed = hbuf(S, dtype=torch.int64)
         self.h_step = hbuf(S, dtype=torch.int64)
         self.h_pen = hbuf(S, dtype=torch.float32)
+        # row maps of stateful models: block-table row of each token, where each token's
+        # previous-token input lives (ops.token_shift), each sequence's last row and state slot
+        self.h_tseq, self.h_ssrc, self.h_srow, self.h_sslot = hbuf(T), hbuf(T), hbuf(S), hbuf(S)
         self._np = [b.numpy() for b in (self.h_ids, self.h_pos, self.h_slots, self.h_cu,
                                          self.h_ctx, self.h_bt, self.h_sid, self.h_smp)]
         (self.n_temp, self.n_topk, self.n_topp, self.n_seed, self.n_step, self.n_pen) = (
@@ -234,6 +258,7 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         self.d_seed = dbuf(S, dtype=torch.int64)
         self.d_step = dbuf(S, dtype=torch.int64)
         self.d_pen = dbuf(S, dtype=torch.float32)
+        self.d_tseq, self.d_ssrc, self.d_srow, self.d_sslot = dbuf(T), dbuf(T), dbuf(S), dbuf(S)
         self.d_tok = dbuf(S)
         self.d_lp = dbuf(S, dtype=torch.float32)
         self.d_tap = dbuf(S, self.mcfg.vocab_size, dtype=torch.float32) if cfg.logits_tap else None
@@ -243,7 +268,8 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         self.step_hook: Optional[Callable[["LLMEngine", int, List[int]], Optional[List[int]]]] = None
         self.decode_ws = ops.DecodeWorkspace(S, self.model.hq, self.model.hkv, cfg.max_model_len,
                                              dev, cfg.decode_pages_per_part, D=self.model.D,
-                                             kv_fp8=cfg.kv_cache_dtype == "fp8") if self.gpu else None
+                                             kv_fp8=cfg.kv_cache_dtype == "fp8") if (
+            self.gpu and getattr(self.model, "uses_decode_workspace", True)) else None
         if self.gpu and self.mcfg.is_moe:
             # this engine's own routing buffers, sized for its largest step before any
             # hipGraph capture (graphs keep pointing at them for the engine's lifetime)
@@ -350,6 +376,8 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
                     self.h_topk, self.h_topp, self.h_seed, self.h_step, self.h_pen, self.h_gidx, self.h_gprev]
             if self._mg_ok:
                 bufs += [self.h_ctxd, self.h_items, self.h_nitems, self.h_sidx]
+            if self.stateful:
+                bufs += [self.h_tseq, self.h_ssrc, self.h_srow, self.h_sslot]
             self._stager = PackedUpload(self.device, sum(b.numel() * b.element_size() + 16 for b in bufs))
         if self.gpu and cfg.use_graphs:
             self._capture_graphs()
@@ -533,6 +561,8 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         t_sched = time.perf_counter()
         kind, n, ntok = self.sched.schedule(ids, pos, sl, cu, ctx, bt, sid, smp)
         nd = n if kind == 2 else (self.sched.last_num_decode() if kind == 3 else 0)
+        if self.stateful and kind:
+            self._fill_row_maps(n, ntok)
         if _KV_SHARE_STATS and nd:   # diagnostics: KV pages the decode rows share (prefix cache)
             nb = (ctx[:nd] + 63) // 64
             refs = np.concatenate([bt[i, :nb[i]] for i in range(nd)])
@@ -748,6 +778,28 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         self.h_topp[n:bs] = 1.0
         self.h_step[n:bs] = 0
         self.h_seed[n:bs] = 0
+        if self.stateful:   # one token per row: no state read, no state write, block-table row = row
+            self.h_ssrc[n:bs] = -1
+            self.h_srow[n:bs] = -1
+            self.h_sslot[n:bs] = -1
+            self.h_tseq[n:bs] = torch.arange(n, bs, dtype=torch.int32)
+
+    def _fill_row_maps(self, n: int, ntok: int) -> None:
+        """Row maps of a scheduled step for models with per-sequence state: ``tok_seq`` (block-
+        table row of every token), ``shift_src`` (where the previous token's layer input is: the
+        row before, zeros at position 0, else the sequence's state slot), and per sequence its
+        last token row and state slot (what the step leaves in the slot)."""
+        pos, cu, sid = self._np[1], self._np[3], self._np[6]
+        tseq, ssrc, srow, sslot = (b.numpy() for b in (self.h_tseq, self.h_ssrc, self.h_srow, self.h_sslot))
+        self.sched.state_slots(sid, n, sslot)
+        q = np.diff(cu[: n + 1])
+        tseq[:ntok] = np.repeat(np.arange(n, dtype=np.int32), q)
+        src = np.arange(-1, ntok - 1, dtype=np.int32)
+        first = cu[:n][q > 0]
+        src[first] = -(sslot[:n][q > 0] + 2)
+        src[pos[:ntok] == 0] = -1
+        ssrc[:ntok] = src
+        srow[:n] = np.where(q > 0, cu[1: n + 1] - 1, -1)
 
     def _finalize(self, pend: dict) -> List[Request]:
         if pend["ev"] is not None:
@@ -902,6 +954,9 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         m = AttnMeta(kind=kind, slots=self.d_slots[:ntok], cu_q=self.d_cu[: n + 1],
                      ctx_lens=self.d_ctx[:n], block_tables=self.d_bt[:n], max_q_len=max_q,
                      max_ctx=max_ctx, decode_ws=self.decode_ws)
+        if self.stateful:
+            m.tok_seq, m.shift_src = self.d_tseq[:ntok], self.d_ssrc[:ntok]
+            m.state_rows, m.state_slots = self.d_srow[:n], self.d_sslot[:n]
         if nd:
             # mixed step: rows [0, nd) decode, the rest prefill with its own cu_seqlens
             m.kind, m.n_decode, m.max_ctx = "mixed", nd, self.cfg.max_model_len
@@ -920,6 +975,9 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
                 (self.h_temp, self.d_temp, npr), (self.h_topk, self.d_topk, npr), (self.h_topp, self.d_topp, npr),
                 (self.h_seed, self.d_seed, npr), (self.h_step, self.d_step, npr), (self.h_pen, self.d_pen, npr)]
         segs += list(extra)
+        if self.stateful:
+            segs += [(self.h_tseq, self.d_tseq, ntok), (self.h_ssrc, self.d_ssrc, ntok),
+                     (self.h_srow, self.d_srow, n), (self.h_sslot, self.d_sslot, n)]
         self._staged_src = None
         if src is not None and len(src[0]):
             k = len(src[0])
@@ -1083,6 +1141,75 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
         ops.sample(logits, self.d_temp[:bs], self.d_topk[:bs], self.d_topp[:bs],
                    self.d_seed[:bs], self.d_step[:bs], None, None,
                    out_tok=self.d_tok[:bs], out_lp=self.d_lp[:bs])
+
+    # ------------------------------------------------------------------ replay of a recorded schedule
+    def replay_step(self, rows: Sequence[Tuple[int, Sequence[int], Sequence[int]]], finished: Sequence[int] = (),
+                    layer_tap: Optional[list] = None) -> Optional[torch.Tensor]:
+        """Run one step whose rows are given instead of chosen: ``rows`` = [(sequence id, its next
+        tokens, places among them whose logits are wanted)]. A sequence is admitted at its first
+        row, may skip steps, and its pages and state slot are given back once it is listed in
+        ``finished``. The step is laid out by the native scheduler (``schedule_rows``: pages on
+        demand, single-token continuations first), uploaded and run like any other step of this
+        engine (decode-only steps replay the captured decode graph when there is one), and
+        nothing is sampled. Returns the fp32 logits [wanted, vocab] in the order of ``rows``
+        (None when nothing is wanted)."""
+        with self.lock:
+            if self._pending is not None:
+                pend, self._pending = self._pending, None
+                self._finalize(pend)
+            live = self._replay_live = getattr(self, "_replay_live", set())
+            ids, counts = [], []
+            for rid, toks, _ in rows:
+                toks = [int(t) for t in toks]
+                if not toks:
+                    raise ValueError("a replayed row needs at least one token")
+                if rid in live:
+                    self.sched.extend(rid, toks)
+                else:
+                    self.sched.add(rid, toks, 0)
+                    live.add(rid)
+                ids.append(int(rid))
+                counts.append(len(toks))
+            logits = None
+            if ids:
+                if self._up_ev is not None:
+                    self._up_ev.synchronize()
+                kind, n, ntok = self.sched.schedule_rows(ids, counts, *self._np)
+                nd = n if kind == 2 else (self.sched.last_num_decode() if kind == 3 else 0)
+                if self.stateful:
+                    self._fill_row_maps(n, ntok)
+                cu, sid = self._np[3], self._np[6]
+                row_of = {int(x): i for i, x in enumerate(sid[:n].tolist())}
+                want = [int(cu[row_of[int(rid)]]) + int(w) for rid, toks, ws in rows for w in ws
+                        if 0 <= int(w) < len(toks)]
+                if sum(len(ws) for _, _, ws in rows) != len(want):
+                    raise ValueError("a wanted place lies outside its row's tokens")
+                self._count(kind, n, ntok, nd)
+                logits = self._replay_forward(kind, n, ntok, nd, want, layer_tap)
+            for rid in finished:
+                self.sched.finish(int(rid))
+                live.discard(rid)
+            return logits
+
+    def _replay_forward(self, kind, n, ntok, nd, want, layer_tap=None):
+        graph = (kind == 2 and self.graphs and self.d_tap is not None and layer_tap is None
+                 and next((b for b in sorted(self.graphs) if b >= n), None))
+        if graph:
+            self._pad_rows(n, graph)
+            self._pad_params(0, graph)
+            self._upload(graph, graph)
+            self.graphs[graph].replay()
+            return self.d_tap.index_select(0, torch.tensor(want, device=self.device)).clone() if want else None
+        self._upload(n, ntok)
+        cu = self._np[3][: n + 1]
+        if kind == 2:
+            meta = self._meta("decode", n, n, 1, self.cfg.max_model_len)
+        else:
+            meta = self._meta("prefill", n, ntok, int((cu[nd + 1:] - cu[nd:-1]).max()), int(self._np[4][:n].max()), nd)
+        idx = torch.tensor(want if want else [ntok - 1], dtype=torch.int64).to(self.device)
+        kw = {"layer_tap": layer_tap} if layer_tap is not None else {}
+        h = self.model.forward(self.d_ids[:ntok], self.d_pos[:ntok], meta, idx, **kw)
+        return self.model.logits(h) if want else None
 
     # ------------------------------------------------------------------ convenience
     def run_until_done(self, reqs: Optional[List[Request]] = None) -> None:

@@ -28,6 +28,8 @@ class StepGraphMixin:
         c, m = self.cfg, self.model
         if not c.mixed_graphs or not (self.gpu and c.use_graphs or c.graph_eager):
             return False
+        if not getattr(m, "supports_step_graphs", True):
+            return False
         self._pf_impl = 2 if (m.D == 128 and m.kv_dtype == "auto" and self.max_blocks <= 1024) else 1
         self._pf_seq_min = int(os.environ.get("NGA_PF_SEQ_MIN", "384"))   # _graph_pf_seq; 0 = off
         return (self.p.pp_size == 1 and not c.sequence_parallel and not m.split_mixed and m.D in (64, 128, 256)

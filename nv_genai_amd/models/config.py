@@ -261,3 +261,111 @@ def llama_config(name_or_cfg, **overrides) -> LlamaConfig:
 def encoder_config(name_or_cfg, **overrides) -> EncoderConfig:
     cfg = ENCODER_PRESETS[name_or_cfg] if isinstance(name_or_cfg, str) else name_or_cfg
     return replace(cfg, **overrides) if overrides else cfg
+
+
+# ---------------------------------------------------------------------------------------------
+# Layer-list decoders: config.json lists the blocks one by one, each with its own mixer sizes.
+@dataclass(frozen=True)
+class SigmoidAttentionSpec:
+    """Mixer ``attention`` of the Bidasun design: un-normalised sigmoid attention with a
+    logarithmic distance term, a sliding window that keeps the first tokens, whole-projection
+    q / k RMS norm and an output gate (``ops.sigmoid_attention``)."""
+
+    heads: int
+    kv_heads: int
+    dim: int            # per-head q / k size
+    vdim: int           # per-head v size
+    scale: float
+    window: int         # i sees j when i - j < window ...
+    keep_first: int     # ... or j < keep_first
+
+
+@dataclass(frozen=True)
+class DenseMlpSpec:
+    ff: int
+    kind: str = "dense"     # down(gelu_tanh(gate x) * (up x))
+
+
+@dataclass(frozen=True)
+class BlockSpec:
+    type: str                              # mixer kind; "attention" -> SigmoidAttentionSpec
+    mixer: SigmoidAttentionSpec
+    mlp: Optional[DenseMlpSpec] = None     # None: the block has no feed-forward
+
+
+@dataclass(frozen=True)
+class BidasunConfig:
+    """Bidasun: post-norm blocks (x += norm(mixer(shift(x))), x += norm(ff(x))) on an fp32
+    residual stream, learned positions, token shift in front of every mixer. Every size and
+    constant comes from the model folder's config.json (:meth:`from_dict`)."""
+
+    name: str = "bidasun"
+    vocab_size: int = 512
+    hidden: int = 128
+    max_position: int = 1024
+    eps: float = 1e-5
+    blocks: tuple = ()
+    arch: str = "bidasun"
+    bos_id: int = 0
+    eos_ids: tuple = ()
+    chat_format: str = "plain"
+    is_moe: bool = False
+
+    @property
+    def layers(self) -> int:
+        return len(self.blocks)
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "bidasun") -> "BidasunConfig":
+        blocks = []
+        for i, b in enumerate(d["layers"]):
+            if b["type"] != "attention":
+                raise ValueError(f"layer {i}: unknown mixer type {b['type']!r}")
+            m = b["mixer"]
+            mixer = SigmoidAttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                         vdim=int(m["vdim"]), scale=float(m["scale"]),
+                                         window=int(m["mask"]["size"]), keep_first=int(m["mask"]["keep_first"]))
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError(f"layer {i}: {mixer.heads} heads over {mixer.kv_heads} kv heads")
+            mlp = b.get("mlp")
+            if mlp is not None:
+                if mlp.get("kind", "dense") != "dense":
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {mlp['kind']!r}")
+                mlp = DenseMlpSpec(ff=int(mlp["ff"]))
+            blocks.append(BlockSpec(type="attention", mixer=mixer, mlp=mlp))
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]),
+                   max_position=int(d["max_positions"]), eps=float(d["norm"]["eps"]), blocks=tuple(blocks))
+
+    def to_json_dict(self) -> dict:
+        """The config.json form (inverse of :meth:`from_dict`)."""
+        return {"architecture": "Bidasun", "vocab": self.vocab_size, "width": self.hidden,
+                "max_positions": self.max_position, "norm": {"eps": self.eps},
+                "layers": [{"type": b.type,
+                            "mixer": {"heads": b.mixer.heads, "kv_heads": b.mixer.kv_heads, "dim": b.mixer.dim,
+                                      "vdim": b.mixer.vdim, "scale": b.mixer.scale,
+                                      "mask": {"size": b.mixer.window, "keep_first": b.mixer.keep_first}},
+                            "mlp": None if b.mlp is None else {"kind": b.mlp.kind, "ff": b.mlp.ff}}
+                           for b in self.blocks]}
+
+    def num_params(self) -> int:
+        n = (2 * self.vocab_size + self.max_position + 1) * self.hidden
+        for b in self.blocks:
+            m = b.mixer
+            nq, nk, nv = m.heads * m.dim, m.kv_heads * m.dim, m.kv_heads * m.vdim
+            n += self.hidden * (nq + nk + nv + 2 * m.heads * m.vdim) + nq + nk + 3 * m.heads + 2 * self.hidden
+            if b.mlp is not None:
+                n += 3 * self.hidden * b.mlp.ff + self.hidden
+        return n
+
+    def to_dict(self):
+        return asdict(self)
+
+
+def bidasun_uniform(layers: int, hidden: int, heads: int, kv_heads: int, dim: int, vdim: int, ff: int,
+                    window: int, keep_first: int, vocab_size: int = 32768, max_position: int = 8192,
+                    scale: Optional[float] = None, eps: float = 1e-5, name: str = "bidasun") -> BidasunConfig:
+    """A Bidasun config whose blocks are all alike (benchmarks, tests)."""
+    m = SigmoidAttentionSpec(heads, kv_heads, dim, vdim, dim ** -0.5 if scale is None else scale, window, keep_first)
+    blk = BlockSpec("attention", m, DenseMlpSpec(ff) if ff else None)
+    return BidasunConfig(name=name, vocab_size=vocab_size, hidden=hidden, max_position=max_position, eps=eps,
+                         blocks=(blk,) * layers)

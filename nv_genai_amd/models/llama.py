@@ -72,6 +72,13 @@ class AttnMeta:
     pf_ks: int = 1
     pf_impl: int = 2    # 2: 32x32 kernel (bf16 head_dim-128 pages), 1: 16x16 kernel
     pf_seq: bool = False  # the work list after the decode attention on the main stream
+    # models with per-sequence state (engine row maps): block-table row of every token, source
+    # of every token's previous-token input (ops.token_shift), and per sequence the last token
+    # row of this step and the state slot it is saved to
+    tok_seq: Optional[torch.Tensor] = None
+    shift_src: Optional[torch.Tensor] = None
+    state_rows: Optional[torch.Tensor] = None
+    state_slots: Optional[torch.Tensor] = None
 
 
 class LlamaModel:

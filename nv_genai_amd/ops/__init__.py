@@ -310,6 +310,101 @@ def rope_cache_(qkv, pos, cos_sin, slots, kc, vc, Hq: int, Hkv: int, D: int,
 
 
 # ------------------------------------------------------------------------- attention
+# ------------------------------------------------------------------------- post-norm fp32 residual rows
+def embed_pos(ids: torch.Tensor, pos: torch.Tensor, embed: torch.Tensor, ptab: torch.Tensor) -> torch.Tensor:
+    """fp32 residual rows: token embedding plus the learned position row (tables bf16 or fp32)."""
+    if not _gpu(embed):
+        return ref.embed_pos(ids, pos, embed, ptab)
+    x = torch.empty(ids.numel(), embed.shape[1], dtype=torch.float32, device=embed.device)
+    kernels().embed_pos(x, ids, pos, embed, ptab)
+    return x
+
+
+def rmsnorm_residual_(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float,
+                      cast_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Post-norm residual step on an fp32 stream: ``x += rmsnorm(y) * w`` in place (statistic and
+    sum in fp32; ``w`` fp32). ``cast_out`` (activation dtype, [T, H]) receives a copy of the new
+    x for the next GEMM."""
+    if not _gpu(x):
+        return ref.rmsnorm_residual_(x, y, w, eps, cast_out)
+    kernels().rmsnorm_residual(x, y, w, float(eps), cast_out)
+    return x
+
+
+def rmsnorm_f32(x: torch.Tensor, w: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
+                dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """RMS norm of fp32 rows (all, or those listed in ``rows``), written in ``dtype``."""
+    if not _gpu(x):
+        return ref.rmsnorm_f32(x, w, eps, rows, dtype)
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty(n, x.shape[1], dtype=dtype, device=x.device)
+    kernels().rmsnorm_f32(out, x, rows, w, float(eps))
+    return out
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, src: torch.Tensor, state: torch.Tensor,
+                dtype: torch.dtype) -> torch.Tensor:
+    """Token shift: ``h[t] = x[t] + (prev(t) - x[t]) * mu`` with prev(t) the input one token
+    earlier. ``src[t]`` says where it is: >= 0 a row of ``x`` (same step), -1 zeros (first token
+    of a sequence), <= -2 row ``-(src + 2)`` of ``state`` [slots, H] (the step before)."""
+    if not _gpu(x):
+        return ref.token_shift(x, mu, src, state, dtype)
+    h = torch.empty(x.shape, dtype=dtype, device=x.device)
+    kernels().token_shift(h, x, mu, src, state)
+    return h
+
+
+def shift_save_(state: torch.Tensor, x: torch.Tensor, last_row: torch.Tensor, slot: torch.Tensor) -> torch.Tensor:
+    """``state[slot[i]] = x[last_row[i]]``: every sequence's last input row of this step becomes
+    its token-shift state (negative slot or row: skipped)."""
+    if not _gpu(x):
+        return ref.shift_save_(state, x, last_row, slot)
+    kernels().shift_save(state, x, last_row, slot)
+    return state
+
+
+def glu_gelu_tanh(x: torch.Tensor) -> torch.Tensor:
+    """[T, 2F] = [gate | up] -> gelu_tanh(gate) * up; bf16 or fp32, any F (the 8-wide bf16
+    kernel when it fits)."""
+    if not _gpu(x):
+        return ref.gelu_tanh_mul(x)
+    F = x.shape[1] // 2
+    if x.dtype == torch.bfloat16 and F % 8 == 0:
+        return gelu_tanh_mul(x)
+    out = torch.empty(x.shape[0], F, dtype=x.dtype, device=x.device)
+    kernels().glu_gelu_tanh(out, x)
+    return out
+
+
+# ------------------------------------------------------------------------- gated sigmoid attention
+def qk_norm_cache_(proj, qw, kw, eps, slots, kc, vc, Hq: int, Hkv: int, dk: int, dv: int):
+    """Whole-projection q / k RMS norm (one statistic over all heads of q, one over all of k;
+    fp32 weights per element) in place on the [q | k | v | ...] projection rows, and the paged
+    write of the normalised k and of v: K [blocks, Hkv, 64, dk], V^T [blocks, Hkv, dv, 64]."""
+    if not _gpu(proj):
+        return ref.qk_norm_cache_(proj, qw, kw, eps, slots, kc, vc, Hq, Hkv, dk, dv)
+    kernels().qk_norm_cache(proj, qw, kw, float(eps), slots, kc, vc, Hq, Hkv, dk, dv)
+    return proj
+
+
+def sigmoid_attention(q, gate, kc, vc, block_tables, tok_seq, pos, Hq: int, Hkv: int, dk: int, dv: int,
+                      scale: float, window: int, keep_first: int, r1, r2, pb, out=None):
+    """Gated sigmoid attention of token rows (prompt portions and decode rows alike) over the
+    paged cache: weight of key j for the query at position i is
+    ``sigmoid(q.k * scale - r1 * ln(1 + r2 * (i - j)) + pb)`` when ``j <= i and (i - j < window
+    or j < keep_first)``, else 0; no normalisation over keys; the head outputs are multiplied
+    by ``sigmoid(gate)``. ``tok_seq[t]`` is the block-table row of token t, ``pos[t]`` its
+    position (negative: padding row, zeros out)."""
+    if not _gpu(q):
+        return ref.sigmoid_attention(q, gate, kc, vc, block_tables, tok_seq, pos, Hq, Hkv, dk, dv, scale, window,
+                                     keep_first, r1, r2, pb)
+    if out is None:
+        out = torch.empty(q.shape[0], Hq * dv, dtype=q.dtype, device=q.device)
+    kernels().sigmoid_attention(out, q, gate, kc, vc, block_tables, tok_seq, pos, Hq, Hkv, dk, dv, float(scale),
+                                int(window), int(keep_first), r1, r2, pb)
+    return out
+
+
 class DecodeWorkspace:
     """Split-K partition buffers for decode attention, sized for (max_seqs, Hq, max_ctx).
 

@@ -431,3 +431,85 @@ def quant_fp8_rows(x, mode: int, Mp: int):
     sp = torch.ones(Mp, 1)
     sp[:M] = s
     return y, sp
+
+
+# ------------------------------------------------------------------------- post-norm fp32 residual rows
+def embed_pos(ids, pos, embed, ptab):
+    """fp32 rows embed[id] + ptab[pos]."""
+    return embed[ids.long()].float() + ptab[pos.long()].float()
+
+
+def rmsnorm_residual_(x, y, w, eps, cast_out=None):
+    """x (fp32, in place) += y * rsqrt(mean(y^2) + eps) * w; ``cast_out`` takes a copy of x."""
+    yf = y.float()
+    x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * w)
+    if cast_out is not None:
+        cast_out.copy_(x)
+    return x
+
+
+def rmsnorm_f32(x, w, eps, rows=None, dtype=torch.float32):
+    xs = x if rows is None else x.index_select(0, rows)
+    return (xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + eps) * w).to(dtype)
+
+
+def token_shift(x, mu, src, state, dtype):
+    """h[t] = x[t] + (prev - x[t]) * mu; prev = x[src] (src >= 0), zeros (-1) or state[-(src + 2)]."""
+    s = src.long()
+    prev = torch.zeros_like(x)
+    rows = s >= 0
+    prev[rows] = x[s[rows]]
+    st = s <= -2
+    prev[st] = state[-(s[st] + 2)]
+    return (x + (prev - x) * mu).to(dtype)
+
+
+def shift_save_(state, x, last_row, slot):
+    ok = (slot >= 0) & (last_row >= 0)
+    state[slot[ok].long()] = x[last_row[ok].long()]
+    return state
+
+
+def qk_norm_cache_(proj, qw, kw, eps, slots, kc, vc, Hq, Hkv, dk, dv):
+    """RMS norm over the whole q and the whole k projection (q written back in place), then the
+    paged write of k and v: K [blocks, Hkv, 64, dk], V^T [blocks, Hkv, dv, 64]."""
+    nq, nk, nv = Hq * dk, Hkv * dk, Hkv * dv
+    q, k = proj[:, :nq].float(), proj[:, nq:nq + nk].float()
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw
+    k = (k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw).to(proj.dtype)
+    proj[:, :nq] = q.to(proj.dtype)
+    sl = slots.long()
+    ok = sl >= 0
+    BS = kc.shape[2]
+    blk, off = sl[ok] // BS, sl[ok] % BS
+    kc[blk, :, off, :] = k[ok].view(-1, Hkv, dk)
+    vc[blk, :, :, off] = proj[ok, nq + nk:nq + nk + nv].reshape(-1, Hkv, dv)
+    return proj
+
+
+def sigmoid_attention(q, gate, kc, vc, block_tables, tok_seq, pos, Hq, Hkv, dk, dv, scale, window, keep_first,
+                      r1, r2, pb):
+    """Un-normalised gated sigmoid attention over paged K / V^T with a sliding window that keeps
+    the first tokens; one row at a time (reference)."""
+    T = q.shape[0]
+    out = torch.zeros(T, Hq * dv, dtype=torch.float32, device=q.device)
+    BS = kc.shape[2]
+    rep = Hq // Hkv
+    heads = torch.arange(Hq, device=q.device) // rep
+    for t in range(T):
+        i = int(pos[t])
+        if i < 0:
+            continue
+        bt = block_tables[int(tok_seq[t])]
+        j = torch.arange(i + 1, device=q.device)
+        j = j[(i - j < window) | (j < keep_first)]
+        blk, off = bt[j // BS].long(), j % BS
+        k = kc[blk, :, off, :].float()[:, heads]           # [n, Hq, dk]
+        v = vc[blk, :, :, off].float()[:, heads]           # [n, Hq, dv]
+        s = torch.einsum("hd,nhd->hn", q[t].float().view(Hq, dk), k) * scale
+        s = s - r1[:, None] * torch.log1p(r2[:, None] * (i - j).float()[None, :])
+        w = torch.sigmoid(s + pb[:, None])
+        out[t] = torch.einsum("hn,nhd->hd", w, v).reshape(-1)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(q.dtype)
