@@ -1059,6 +1059,40 @@ void sigmoid_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor 
                                 r2.data_ptr<float>(), pb.data_ptr<float>(), f32, cur_stream(q));
 }
 
+
+// prompt portions on the MFMA kernel (bf16; dk, dv in {32, 64, 128}): sequence b owns rows
+// [cu_q[b], cu_q[b + 1]) of q / gate / out, the last ones of its ctx_lens[b] keys
+void sigmoid_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc,
+                               Tensor block_tables, Tensor cu_q, Tensor ctx_lens, int64_t max_q_len, int64_t Hq,
+                               int64_t Hkv, int64_t dk, int64_t dv, double scale, int64_t window, int64_t keep_first,
+                               Tensor r1, Tensor r2, Tensor pb) {
+  CHECK_BF16(q); CHECK_BF16(out); CHECK_CONTIG(out);
+  CHECK_F32(r1); CHECK_F32(r2); CHECK_F32(pb); CHECK_I32(block_tables); CHECK_I32(cu_q); CHECK_I32(ctx_lens);
+  TORCH_CHECK(nga::sigmoid_attention_mfma_supported((int)dk, (int)dv), "sigmoid_attention_prefill: dk, dv in {32, 64, 128}");
+  const int64_t T = q.size(0), B = ctx_lens.numel();
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == Hq * dk && q.stride(0) % 8 == 0 &&
+              (uintptr_t)q.data_ptr() % 16 == 0, "q must be 16-B aligned [T, Hq * dk] rows");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == Hq * dv);
+  TORCH_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && window > 0 && keep_first >= 0 && max_q_len >= 0);
+  TORCH_CHECK(r1.numel() == Hq && r2.numel() == Hq && pb.numel() == Hq);
+  TORCH_CHECK(cu_q.numel() == B + 1 && block_tables.dim() == 2 && block_tables.size(0) >= B);
+  check_sig_pages(q, kc, vc, Hkv, dk, dv);
+  const uint16_t* gp = nullptr;
+  int64_t gs = 0;
+  if (gate.has_value()) {
+    CHECK_BF16(*gate);
+    TORCH_CHECK(gate->dim() == 2 && gate->size(0) == T && gate->size(1) == Hq * dv && gate->stride(1) == 1 &&
+                gate->stride(0) % 4 == 0 && (uintptr_t)gate->data_ptr() % 8 == 0, "gate must be 8-B aligned rows");
+    gp = bfp(*gate);
+    gs = gate->stride(0);
+  }
+  nga::launch_sigmoid_attention_mfma(bfp(out), bfp(q), q.stride(0), gp, gs, bfp(kc), bfp(vc),
+                                     block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
+                                     cu_q.data_ptr<int32_t>(), ctx_lens.data_ptr<int32_t>(), (int)B, (int)max_q_len,
+                                     (int)Hq, (int)Hkv, (int)dk, (int)dv, (float)scale, (int)window, (int)keep_first,
+                                     r1.data_ptr<float>(), r2.data_ptr<float>(), pb.data_ptr<float>(), cur_stream(q));
+}
+
 }  // namespace
 
 
@@ -1120,6 +1154,8 @@ PYBIND11_MODULE(_C, m) {
   m.def("glu_gelu_tanh", checked("glu_gelu_tanh", &glu_gelu_tanh));
   m.def("qk_norm_cache", checked("qk_norm_cache", &qk_norm_cache));
   m.def("sigmoid_attention", checked("sigmoid_attention", &sigmoid_attention));
+  m.def("sigmoid_attention_prefill", checked("sigmoid_attention_prefill", &sigmoid_attention_prefill));
+  m.def("sigmoid_attention_mfma_supported", [](int64_t dk, int64_t dv) { return nga::sigmoid_attention_mfma_supported((int)dk, (int)dv); });
   m.def("silu_mul", checked("silu_mul", &silu_mul));
   m.def("bias_gelu", checked("bias_gelu", &bias_gelu));
   m.def("rope_cache", checked("rope_cache", &rope_cache));

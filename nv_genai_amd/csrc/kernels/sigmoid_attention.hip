@@ -17,6 +17,8 @@
 //
 // Pages: K [blocks, Hkv, 64, dk], V^T [blocks, Hkv, dv, 64] (T = bf16 or fp32). Scores, the
 // distance term, the sigmoid and the accumulation are fp32 in every form.
+#include <cstdlib>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -152,6 +154,169 @@ __global__ void __launch_bounds__(64) sigmoid_attention_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// MFMA form for prompt portions (bf16). Workgroup = 4 waves = 64 query rows of one sequence and
+// one query head; each wave owns 16 rows, the 16 columns of its mfma_f32_16x16x32_bf16 tiles.
+// Per 64-key page the workgroup stages K [64][DK] and V^T [DV][64] in LDS (16-B chunks XOR-
+// swizzled by row), then every wave computes S^T = K . Q^T with the key rows permuted so that
+// lane (query, h) ends up holding keys 32g + 8h .. + 7 of the page in its accumulators — which is
+// exactly the B operand of O^T += V^T . W^T, so the weights never move between lanes. Between
+// the two products the weights are formed in fp32 on the VALU (scale, distance term, bias,
+// sigmoid, mask). Pages visited: those holding kept first tokens below the block's window, then
+// the pages the block's windows cover; everything between is skipped.
+__device__ __forceinline__ int sg_row_swz(int row) { return (row & 3) | (((row >> 3) & 3) << 2); }
+
+struct SigMfmaParams {
+  uint16_t* out;             // [T, Hq * DV]
+  const uint16_t* q;         // row stride q_stride, head h at h * DK
+  const uint16_t* gate;      // row stride g_stride, head h at h * DV (nullptr: none)
+  const uint16_t* kc;
+  const uint16_t* vc;
+  const int32_t* block_tables;
+  const int32_t* cu_q;       // [B + 1] token rows of each sequence in this launch
+  const int32_t* ctx_lens;   // [B] keys of each sequence after this step (its rows are the last ones)
+  const float* r1;
+  const float* r2;
+  const float* pb;
+  int64_t q_stride, g_stride;
+  int max_blocks, Hq, Hkv, window, keep_first;
+  float scale;
+};
+
+template <int DK, int DV>
+__global__ void __launch_bounds__(256) sigmoid_attention_mfma_kernel(const SigMfmaParams P) {
+  constexpr int KT = 64;
+  constexpr int NCH_K = DK / 8;
+  constexpr int DS = DK / 32;
+  constexpr int DT = DV / 16;
+  constexpr int PER_K = DK / 32, PER_V = DV / 32;   // 16-B chunks per thread per page
+  constexpr int SWS = NCH_K >= 16 ? 0 : NCH_K == 8 ? 1 : 2;
+  __shared__ __attribute__((aligned(16))) uint16_t k_s[KT * DK];
+  __shared__ __attribute__((aligned(16))) uint16_t v_s[DV * KT];
+  const int tile = blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
+  const int q0 = P.cu_q[b], qlen = P.cu_q[b + 1] - q0;
+  if (tile * 64 >= qlen) return;
+  const int ctx = P.ctx_lens[b];
+  const int kvh = hq / (P.Hq / P.Hkv);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, h = lane >> 4;
+  const int W = P.window, keep = P.keep_first;
+
+  int r = tile * 64 + w * 16 + col;
+  const bool row_ok = r < qlen;
+  if (!row_ok) r = qlen - 1;
+  const int qpos = ctx - qlen + r;
+  bf16x8 qf[DS];
+  {
+    const uint16_t* qp = P.q + (int64_t)(q0 + r) * P.q_stride + (int64_t)hq * DK;
+#pragma unroll
+    for (int s2 = 0; s2 < DS; ++s2) qf[s2] = as_bf16x8(load8(qp + 32 * s2 + 8 * h));
+  }
+  // pages of this block: kept ones below its oldest window start, then [t_first, t_last]
+  const int qpos_lo = ctx - qlen + tile * 64;
+  const int qpos_hi = ctx - qlen + min(qlen - 1, tile * 64 + 63);
+  const int lo_min = max(0, qpos_lo - W + 1);
+  const int t_first = lo_min / KT, t_last = qpos_hi / KT;
+  const int t_keep_end = (min(keep, lo_min) + KT - 1) / KT;
+  const float a1 = P.r1[hq], a2 = P.r2[hq], bias = P.pb[hq];
+
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4)(0.f);
+
+  for (int t = 0; t <= t_last; ++t) {
+    if (t >= t_keep_end && t < t_first) t = t_first;
+    const int64_t blk = P.block_tables[(int64_t)b * P.max_blocks + t];
+    const uint16_t* kp = P.kc + (blk * P.Hkv + kvh) * (int64_t)(KT * DK);
+    const uint16_t* vp = P.vc + (blk * P.Hkv + kvh) * (int64_t)(DV * KT);
+    u16x8 kreg[PER_K], vreg[PER_V];
+#pragma unroll
+    for (int i = 0; i < PER_K; ++i) kreg[i] = load8(kp + (int64_t)(tid + 256 * i) * 8);
+#pragma unroll
+    for (int i = 0; i < PER_V; ++i) vreg[i] = load8(vp + (int64_t)(tid + 256 * i) * 8);
+    __syncthreads();   // the previous page's reads are done
+#pragma unroll
+    for (int i = 0; i < PER_K; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c / NCH_K, ch = c % NCH_K;
+      const int sw = sg_row_swz(row) >> SWS;
+      *reinterpret_cast<u16x8*>(&k_s[row * DK + ((ch ^ sw) * 8)]) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < PER_V; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c / 8, ch = c % 8;
+      *reinterpret_cast<u16x8*>(&v_s[row * KT + ((ch ^ ((row >> 1) & 7)) * 8)]) = vreg[i];
+    }
+    __syncthreads();
+
+    f32x4 sacc[4];
+#pragma unroll
+    for (int tau = 0; tau < 4; ++tau) {
+      const int row = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
+      const int sw = sg_row_swz(row) >> SWS;
+      sacc[tau] = (f32x4)(0.f);
+#pragma unroll
+      for (int s2 = 0; s2 < DS; ++s2) {
+        const int ch = 4 * s2 + h;
+        const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&k_s[row * DK + ((ch ^ sw) * 8)]));
+        sacc[tau] = mfma16(a, qf[s2], sacc[tau]);
+      }
+    }
+    const int kbase = t * KT;
+    bf16x8 pf[2];
+#pragma unroll
+    for (int tau = 0; tau < 4; ++tau)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int key = kbase + 32 * (tau >> 1) + 8 * h + 4 * (tau & 1) + rr;
+        const int dist = qpos - key;
+        const bool ok = dist >= 0 && (dist < W || key < keep);
+        const float z = sacc[tau][rr] * P.scale - a1 * __logf(1.0f + a2 * (float)dist) + bias;
+        const float wv = ok ? __builtin_amdgcn_rcpf(1.0f + __expf(-z)) : 0.f;
+        pf[tau >> 1][4 * (tau & 1) + rr] = (__bf16)wv;
+      }
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const int ch = 4 * g + h;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const int row = 16 * dt + col;
+        const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&v_s[row * KT + ((ch ^ ((row >> 1) & 7)) * 8)]));
+        o[dt] = mfma16(a, pf[g], o[dt]);
+      }
+    }
+  }
+  if (!row_ok) return;
+  uint16_t* op = P.out + (int64_t)(q0 + r) * P.Hq * DV + (int64_t)hq * DV;
+  const uint16_t* gp = P.gate ? P.gate + (int64_t)(q0 + r) * P.g_stride + (int64_t)hq * DV : nullptr;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int d = 16 * dt + 4 * h;
+    u16x4 ov;
+    u16x4 gv;
+    if (gp) gv = *reinterpret_cast<const u16x4*>(gp + d);
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      float v = o[dt][rr];
+      if (gp) v *= sigmoidf_(bf2f(gv[rr]));
+      ov[rr] = f2bf(v);
+    }
+    *reinterpret_cast<u16x4*>(op + d) = ov;
+  }
+}
+
+template <int DK>
+bool launch_sig_mfma_dv(const SigMfmaParams& P, int dv, dim3 grid, hipStream_t stream) {
+  switch (dv) {
+    case 32: sigmoid_attention_mfma_kernel<DK, 32><<<grid, 256, 0, stream>>>(P); return true;
+    case 64: sigmoid_attention_mfma_kernel<DK, 64><<<grid, 256, 0, stream>>>(P); return true;
+    case 128: sigmoid_attention_mfma_kernel<DK, 128><<<grid, 256, 0, stream>>>(P); return true;
+    default: return false;
+  }
+}
+
 }  // namespace
 
 void launch_qk_norm_cache(void* proj, int64_t stride, const float* qw, const float* kw, float eps,
@@ -184,6 +349,30 @@ void launch_sigmoid_attention(void* out, const void* q, int64_t q_stride, const 
         (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)gate, g_stride, (const uint16_t*)kc,
         (const uint16_t*)vc, block_tables, max_blocks, tok_seq, pos, Hq, Hkv, dk, dv, scale, window, keep_first, r1,
         r2, pb);
+}
+
+bool sigmoid_attention_mfma_supported(int dk, int dv) {
+  return (dk == 32 || dk == 64 || dk == 128) && (dv == 32 || dv == 64 || dv == 128);
+}
+
+// Prompt portions on the MFMA kernel: sequence b owns token rows [cu_q[b], cu_q[b + 1]), the last
+// ones of its ctx_lens[b] keys. Row strides and the gate pointer must be 8-byte aligned (checked
+// by the caller together with sigmoid_attention_mfma_supported).
+void launch_sigmoid_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_stride, const uint16_t* gate,
+                                   int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
+                                   const int32_t* block_tables, int max_blocks, const int32_t* cu_q,
+                                   const int32_t* ctx_lens, int B, int max_q_len, int Hq, int Hkv, int dk, int dv,
+                                   float scale, int window, int keep_first, const float* r1, const float* r2,
+                                   const float* pb, hipStream_t stream) {
+  if (B == 0 || max_q_len == 0) return;
+  SigMfmaParams P{out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, r1, r2, pb, q_stride, g_stride,
+                  max_blocks, Hq, Hkv, window, keep_first, scale};
+  const dim3 grid((unsigned)((max_q_len + 63) / 64), (unsigned)Hq, (unsigned)B);
+  bool ok = false;
+  if (dk == 32) ok = launch_sig_mfma_dv<32>(P, dv, grid, stream);
+  else if (dk == 64) ok = launch_sig_mfma_dv<64>(P, dv, grid, stream);
+  else if (dk == 128) ok = launch_sig_mfma_dv<128>(P, dv, grid, stream);
+  if (!ok) abort();   // the caller checks sigmoid_attention_mfma_supported
 }
 
 }  // namespace nga

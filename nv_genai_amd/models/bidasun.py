@@ -59,6 +59,7 @@ class BidasunModel:
         self.k_cache: List[torch.Tensor] = []
         self.v_cache: List[torch.Tensor] = []
         self.shift_state: List[torch.Tensor] = []
+        self.mfma_prefill = True   # prompt portions on the MFMA kernel where it applies (bf16, dims 32 / 64 / 128)
         if weights is None:
             weights = random_weights(cfg, seed, dtype)
         self._load(weights)
@@ -166,9 +167,22 @@ class BidasunModel:
         proj = ops.linear(h, L["wqkvg"])
         ops.qk_norm_cache_(proj, L["qn"], L["kn"], self.cfg.eps, meta.slots, self.k_cache[li], self.v_cache[li],
                            m.heads, m.kv_heads, m.dim, m.vdim)
-        a = ops.sigmoid_attention(proj[:, :nq], proj[:, nq + nk + nv:], self.k_cache[li], self.v_cache[li],
-                                  meta.block_tables, meta.tok_seq, pos, m.heads, m.kv_heads, m.dim, m.vdim,
-                                  m.scale, m.window, m.keep_first, L["r1"], L["r2"], L["pb"])
+        q, gate = proj[:, :nq], proj[:, nq + nk + nv:]
+        kc, vc = self.k_cache[li], self.v_cache[li]
+        args = (m.heads, m.kv_heads, m.dim, m.vdim, m.scale, m.window, m.keep_first, L["r1"], L["r2"], L["pb"])
+        nd = meta.n_decode if meta.kind == "mixed" else 0
+        if meta.kind in ("prefill", "mixed") and self.mfma_prefill and ops.sigmoid_attention_mfma_ok(proj, m.dim, m.vdim):
+            # prompt portions on MFMA tiles; the single-token rows of a mixed step (its first
+            # n_decode rows) on the row kernel, into disjoint rows of one output
+            a = torch.empty(proj.shape[0], L["ng"], dtype=proj.dtype, device=proj.device)
+            if nd:
+                ops.sigmoid_attention(q[:nd], gate[:nd], kc, vc, meta.block_tables, meta.tok_seq[:nd], pos[:nd], *args,
+                                      out=a[:nd])
+            ops.sigmoid_attention_prefill(q[nd:], gate[nd:], kc, vc, meta.block_tables[nd:],
+                                          meta.cu_q_prefill if nd else meta.cu_q, meta.ctx_lens[nd:],
+                                          meta.max_q_len, *args, out=a[nd:])
+        else:
+            a = ops.sigmoid_attention(q, gate, kc, vc, meta.block_tables, meta.tok_seq, pos, *args)
         return ops.linear(a, L["wo"])
 
     def forward(self, ids: torch.Tensor, pos: torch.Tensor, meta: AttnMeta,

@@ -405,6 +405,36 @@ def sigmoid_attention(q, gate, kc, vc, block_tables, tok_seq, pos, Hq: int, Hkv:
     return out
 
 
+def sigmoid_attention_mfma_ok(q: torch.Tensor, dk: int, dv: int) -> bool:
+    """The MFMA prompt kernel takes bf16 GPU rows with dk, dv in {32, 64, 128}."""
+    return _gpu(q) and q.dtype == torch.bfloat16 and dk in (32, 64, 128) and dv in (32, 64, 128)
+
+
+def sigmoid_attention_prefill(q, gate, kc, vc, block_tables, cu_q, ctx_lens, max_q_len: int, Hq: int, Hkv: int,
+                              dk: int, dv: int, scale: float, window: int, keep_first: int, r1, r2, pb, out=None):
+    """:func:`sigmoid_attention` of prompt portions on MFMA tiles: sequence b owns token rows
+    ``[cu_q[b], cu_q[b + 1])``, the last ones of its ``ctx_lens[b]`` keys (bf16; see
+    :func:`sigmoid_attention_mfma_ok`). CPU tensors take the row reference."""
+    if not _gpu(q):
+        n = cu_q[1:] - cu_q[:-1]
+        seq = torch.repeat_interleave(torch.arange(n.numel(), dtype=torch.int32), n.long())
+        pos = torch.cat([torch.arange(int(c) - int(k), int(c), dtype=torch.int32) for c, k in zip(ctx_lens, n)])
+        return ref.sigmoid_attention(q, gate, kc, vc, block_tables, seq, pos, Hq, Hkv, dk, dv, scale, window,
+                                     keep_first, r1, r2, pb)
+    if not sigmoid_attention_mfma_ok(q, dk, dv):   # fp32 rows / other head sizes: the row kernel
+        T, dev = q.shape[0], q.device
+        n = (cu_q[1:] - cu_q[:-1]).long()
+        seq = torch.repeat_interleave(torch.arange(n.numel(), device=dev), n, output_size=T)
+        pos = (ctx_lens.long() - n - cu_q[:-1].long())[seq] + torch.arange(T, device=dev)
+        return sigmoid_attention(q, gate, kc, vc, block_tables, seq.int(), pos.int(), Hq, Hkv, dk, dv, scale, window,
+                                 keep_first, r1, r2, pb, out=out)
+    if out is None:
+        out = torch.empty(q.shape[0], Hq * dv, dtype=q.dtype, device=q.device)
+    kernels().sigmoid_attention_prefill(out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, int(max_q_len), Hq, Hkv,
+                                        dk, dv, float(scale), int(window), int(keep_first), r1, r2, pb)
+    return out
+
+
 class DecodeWorkspace:
     """Split-K partition buffers for decode attention, sized for (max_seqs, Hq, max_ctx).
 

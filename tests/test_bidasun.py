@@ -34,6 +34,17 @@ def cfg_dict(width=40, vocab=97, positions=512, layers=None, eps=1e-5):
                         "mlp": None if l["ff"] is None else {"kind": "dense", "ff": l["ff"]}} for l in layers]}
 
 
+def cfg_dict_tiles():
+    """Head sizes the MFMA prompt kernel takes (32 / 64 / 128), unequal per block."""
+    return cfg_dict(width=48, layers=[
+        dict(heads=2, kv_heads=1, dim=32, vdim=64, window=70, keep_first=3, scale=0.2, ff=40),
+        dict(heads=3, kv_heads=3, dim=64, vdim=32, window=9, keep_first=0, scale=0.15, ff=None),
+        dict(heads=2, kv_heads=2, dim=128, vdim=128, window=130, keep_first=66, scale=0.1, ff=24)])
+
+
+CFGS = {"odd": cfg_dict, "tiles": cfg_dict_tiles}
+
+
 def build(device, dtype="float32", seed=0, pages=24, seqs=4, cd=None, graphs=None, **eng):
     cd = cd or cfg_dict()
     cfg = BidasunConfig.from_dict(cd)
@@ -187,7 +198,7 @@ def test_one_key_stands_out(device, dtype):
     part of a prompt portion and as a single decode row."""
     tdt = getattr(torch, dtype)
     Hq = G = 1
-    dk, dv, W, keep, T = 8, 8, 37, 5, 200
+    dk, dv, W, keep, T = 32, 32, 37, 5, 200
     r1, r2 = torch.tensor([0.0]), torch.tensor([0.3])
     pb = torch.tensor([-30.0])
     bt_row = [3, 1, 6, 2]
@@ -206,17 +217,57 @@ def test_one_key_stands_out(device, dtype):
             for rows in (list(range(max(0, i - 2), i + 1)), [i]):     # a portion ending at i / i alone
                 pos = torch.tensor(rows, dtype=torch.int32, device=device)
                 seq = torch.zeros(len(rows), dtype=torch.int32, device=device)
-                got = ops.sigmoid_attention(q.reshape(T, -1)[rows].contiguous().to(tdt).to(device), None, kc, vc, bt,
-                                            seq, pos, Hq, G, dk, dv, 1.0, W, keep, r1.to(device), r2.to(device),
-                                            pb.to(device))
+                qr = q.reshape(T, -1)[rows].contiguous().to(tdt).to(device)
+                tail = (Hq, G, dk, dv, 1.0, W, keep, r1.to(device), r2.to(device), pb.to(device))
+                got = ops.sigmoid_attention(qr, None, kc, vc, bt, seq, pos, *tail)
+                if len(rows) > 1:   # the portion through the prompt kernel too (MFMA tiles in bf16 on the GPU)
+                    cu = torch.tensor([0, len(rows)], dtype=torch.int32, device=device)
+                    cx = torch.tensor([i + 1], dtype=torch.int32, device=device)
+                    got2 = ops.sigmoid_attention_prefill(qr, None, kc, vc, bt, cu, cx, len(rows), *tail)
+                    err2 = (got2[-1].double().cpu() - want).abs().max().item()
+                    assert err2 < 1e-2, f"prompt kernel: query {i}, key {j}, visible {vis}: off by {err2}"
                 err = (got[-1].double().cpu() - want).abs().max().item()
                 assert err < 1e-2, f"query {i}, key {j}, visible {vis}: off by {err}"
 
 
-# ---------------------------------------------------------------------------- the model on the engine
 @pytest.mark.parametrize("device,dtype", DTYPES)
-def test_whole_prompt_and_layers(device, dtype):
-    eng, cd, W = build(device, dtype)
+def test_sigmoid_attention_prompt_portions(device, dtype):
+    """The prompt-portion entry point (MFMA tiles for bf16 on the GPU): three sequences whose
+    portions start in the middle of a page, end past a window and differ in length."""
+    torch.manual_seed(4)
+    tdt = getattr(torch, dtype)
+    for Hq, G, dk, dv, W, keep in ((2, 1, 32, 64, 70, 3), (3, 3, 64, 32, 9, 0), (2, 2, 128, 128, 130, 66), (4, 2, 64, 64, 64, 64)):
+        ctxs, qlens = [200, 67, 130], [150, 67, 2]
+        r1, r2, pb = torch.rand(Hq) + 0.5, torch.rand(Hq) * 0.5 + 0.05, torch.randn(Hq) - 1
+        bts = [[4, 0, 7, 9], [1, 2, 11, 11], [3, 5, 6, 11]]
+        nb = 12
+        kc = torch.zeros(nb, G, 64, dk, dtype=tdt, device=device)
+        vc = torch.zeros(nb, G, dv, 64, dtype=tdt, device=device)
+        qs, gs, wants = [], [], []
+        for c, n, bt_row in zip(ctxs, qlens, bts):
+            q, k, v = torch.randn(c, Hq, dk).to(tdt), torch.randn(c, G, dk).to(tdt), torch.randn(c, G, dv).to(tdt)
+            gate = torch.randn(c, Hq * dv).to(tdt)
+            for t in range(c):
+                kc[bt_row[t // 64], :, t % 64, :] = k[t].to(device)
+                vc[bt_row[t // 64], :, :, t % 64] = v[t].to(device)
+            want = O.o_sigmoid_attention(q.double(), k.double(), v.double(), Hq, G, 0.2, W, keep, r1.double(),
+                                         r2.double(), pb.double()).reshape(c, -1) * torch.sigmoid(gate.double())
+            qs.append(q.reshape(c, -1)[c - n:])
+            gs.append(gate[c - n:])
+            wants.append(want[c - n:])
+        cu = torch.tensor([0, 150, 217, 219], dtype=torch.int32, device=device)
+        got = ops.sigmoid_attention_prefill(torch.cat(qs).to(device), torch.cat(gs).to(device), kc, vc,
+                                            torch.tensor(bts, dtype=torch.int32, device=device), cu,
+                                            torch.tensor(ctxs, dtype=torch.int32, device=device), 150, Hq, G, dk, dv,
+                                            0.2, W, keep, r1.to(device), r2.to(device), pb.to(device))
+        close(got, torch.cat(wants), dtype, f"prompt portions {Hq},{G},{dk},{dv},{W},{keep}")
+
+
+# ---------------------------------------------------------------------------- the model on the engine
+@pytest.mark.parametrize("shape", sorted(CFGS))
+@pytest.mark.parametrize("device,dtype", DTYPES)
+def test_whole_prompt_and_layers(device, dtype, shape):
+    eng, cd, W = build(device, dtype, cd=CFGS[shape]())
     toks = tokens(200)
     want, layers = O.o_forward(cd, W, toks)
     tap = []
@@ -228,9 +279,10 @@ def test_whole_prompt_and_layers(device, dtype):
     close(got[:3], O.o_forward(cd, W, toks[:3])[0], dtype, "first tokens")
 
 
+@pytest.mark.parametrize("shape", sorted(CFGS))
 @pytest.mark.parametrize("device,dtype", DTYPES)
-def test_prefill_then_decode_and_portions(device, dtype):
-    eng, cd, W = build(device, dtype)
+def test_prefill_then_decode_and_portions(device, dtype, shape):
+    eng, cd, W = build(device, dtype, cd=CFGS[shape]())
     toks = tokens(230, seed=5)
     want = O.o_forward(cd, W, toks)[0]
     close(replay_cuts(eng, toks, [70]), want, dtype, "prompt then token by token (160 decoded, windows pass)")
@@ -239,12 +291,13 @@ def test_prefill_then_decode_and_portions(device, dtype):
     assert eng.sched.free_blocks() == eng.num_blocks and eng.sched.free_state_slots() == 4
 
 
+@pytest.mark.parametrize("shape", sorted(CFGS))
 @pytest.mark.parametrize("device,dtype", DTYPES)
-def test_mixed_batches_and_reuse(device, dtype):
+def test_mixed_batches_and_reuse(device, dtype, shape):
     """Four unequal requests interleaved (portions beside single tokens, a request that skips
     steps), in a pool that only holds the live ones: pages and slots are freed and used again by
     requests that start later. Every request must equal its run alone (the oracle)."""
-    eng, cd, W = build(device, dtype, pages=9, seqs=3)
+    eng, cd, W = build(device, dtype, pages=9, seqs=3, cd=CFGS[shape]())
     reqs = {i: tokens(n, seed=10 + i) for i, n in enumerate((150, 65, 1, 200, 129, 64, 3))}
     want = {i: O.o_forward(cd, W, t)[0] for i, t in reqs.items()}
     got = {i: [] for i in reqs}
