@@ -104,7 +104,9 @@ def parse(argv=None):
                     help="tensor-parallel ranks per replica (N / tp replicas)")
     ap.add_argument("--sharded-index", action="store_true",
                     help="stripe each replica's index over its tp ranks (broadcast + all-gather merge)")
-    ap.add_argument("--workload", choices=("rag", "agent"), default="rag",
+    ap.add_argument("--design-sizes", default=None,
+                    help="--workload designs: comma list of s, m, l (benchmarks/design_compare.py)")
+    ap.add_argument("--workload", choices=("rag", "agent", "designs"), default="rag",
                     help="agent: query-decomposition agent, one TP=N replica + N-way sharded index")
     ap.add_argument("--kv-cache-fraction", type=float, default=None)
     ap.add_argument("--no-step-graphs", action="store_true",
@@ -309,6 +311,13 @@ def main(argv=None):
     shared = check_devices(args, world_env)
     if args.workload == "agent":
         run_agent(args, world_env, shared)
+        return
+    if args.workload == "designs":
+        # Bidasun beside the equal-size sliding-window Mistral: engine prefill / decode rates and
+        # the attention kernels against their rooflines (one GPU; the default workload is untouched)
+        from benchmarks.design_compare import run as run_designs
+
+        run_designs(args)
         return
     if world_env > 1:
         # one rank per GPU on a shared host: give each rank's tokenizer thread pool (Rust

@@ -1,0 +1,162 @@
+"""Bidasun beside the closest Llama-layout model (Mistral with a sliding window) at equal sizes:
+prefill and decode throughput through the serving engine, and the attention kernels alone with
+their distance from the roofline. Random weights, synthetic token ids.
+
+    python bench.py --workload designs [--design-sizes s,m,l]
+
+Prints one JSON line (``metric: design_compare``); bench.py's default workload is untouched.
+"""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+SIZES = {
+    # name: hidden, heads, kv_heads, head size, ffn, window, layers, prompts x tokens, decode rows x context
+    "s": dict(hidden=1024, heads=8, kv=2, d=128, ffn=2816, window=1024, layers=4, pf=(8, 2048), dec=(64, 2048)),
+    "m": dict(hidden=2048, heads=16, kv=4, d=128, ffn=5632, window=2048, layers=4, pf=(4, 4096), dec=(64, 4096)),
+    "l": dict(hidden=4096, heads=32, kv=8, d=128, ffn=14336, window=4096, layers=2, pf=(2, 8192), dec=(64, 8192)),
+}
+VOCAB = 32768
+PEAK_BF16 = 2.5e15      # dense MFMA flop/s
+PEAK_HBM = 8.0e12       # bytes/s
+PEAK_TRANS = 256 * 16 * 2.4e9   # transcendental lanes/s: 256 CUs x 4 SIMDs x 4 lanes/clk at 2.4 GHz
+
+
+def _engine(kind: str, z: dict, max_len: int, pages: int, seqs: int):
+    from nv_genai_amd.engine.llm_engine import EngineConfig, LLMEngine
+    from nv_genai_amd.models.config import LlamaConfig, bidasun_uniform
+
+    if kind == "bidasun":
+        mcfg = bidasun_uniform(z["layers"], z["hidden"], z["heads"], z["kv"], z["d"], z["d"], z["ffn"], z["window"], 4,
+                               vocab_size=VOCAB, max_position=max_len)
+    else:
+        mcfg = LlamaConfig(name="mistral-eq", arch="mistral", vocab_size=VOCAB, hidden=z["hidden"], layers=z["layers"],
+                           heads=z["heads"], kv_heads=z["kv"], head_dim=z["d"], ffn=z["ffn"],
+                           sliding_window=z["window"], max_position=max_len, rope_theta=1e6, eos_ids=(2,), bos_id=1)
+    cfg = EngineConfig(model=mcfg.name, max_num_seqs=seqs, max_batched_tokens=z["pf"][0] * z["pf"][1],
+                       max_model_len=max_len, kv_cache_blocks=pages, enable_prefix_caching=False, detokenize=False,
+                       use_graphs=True, graph_batch_sizes=(seqs,), mixed_graphs=False, logits_tap=True,
+                       tuned_gemms=False, async_decode=False)
+    return LLMEngine(cfg, device="cuda", model_cfg=mcfg)
+
+
+def _timed(fn, n: int) -> float:
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / n
+
+
+def engine_rates(kind: str, z: dict, steps: int, warmup: int) -> dict:
+    """tokens/s of whole-prompt prefill steps and of decode steps (the captured decode graph)."""
+    nb, L = z["pf"]
+    nd, ctx = z["dec"]
+    max_len = max(L, ctx) + 64 * (steps + warmup + 2)
+    pages = max(nb * -(-L // 64), nd * -(-(ctx + steps + warmup + 2) // 64)) + 8
+    eng = _engine(kind, z, max_len, pages, max(nb, nd))
+    g = torch.Generator().manual_seed(0)
+    rid = [0]
+
+    def prefill():
+        rows = []
+        for _ in range(nb):
+            rid[0] += 1
+            rows.append((rid[0], torch.randint(3, VOCAB, (L,), generator=g).tolist(), [L - 1]))
+        eng.replay_step(rows, [r for r, _, _ in rows])
+
+    for _ in range(warmup):
+        prefill()
+    t_pf = _timed(prefill, steps)
+    # decode: nd sequences of ctx tokens (filled in chunks), then single-token steps
+    ids = list(range(10_000, 10_000 + nd))
+    per = max(1, (nb * L) // ctx)
+    for i in range(0, nd, per):
+        eng.replay_step([(r, torch.randint(3, VOCAB, (ctx,), generator=g).tolist(), []) for r in ids[i:i + per]], [])
+
+    def decode():
+        eng.replay_step([(r, [5], [0]) for r in ids], [])
+
+    for _ in range(warmup):
+        decode()
+    t_dec = _timed(decode, steps)
+    return {"prefill_tok_s": round(nb * L / t_pf), "prefill_ms": round(t_pf * 1e3, 2),
+            "decode_tok_s": round(nd / t_dec), "decode_ms": round(t_dec * 1e3, 3),
+            "decode_graph": bool(eng.graphs)}
+
+
+def kernel_times(z: dict, iters: int = 20) -> dict:
+    """The attention kernels alone on one layer's shapes: time, and the fraction of the roofline
+    (MFMA flops for the prompt kernels, plus the transcendental rate for the sigmoid one, which
+    needs a log, an exp and a reciprocal per score; HBM bytes of the visible pages for decode)."""
+    from nv_genai_amd import ops
+
+    dev, bf = "cuda", torch.bfloat16
+    H, G, D, W = z["heads"], z["kv"], z["d"], z["window"]
+    nb, L = z["pf"]
+    nd, ctx = z["dec"]
+    pages_seq = -(-max(L, ctx) // 64)
+    nseq = max(nb, nd)
+    npg = nseq * pages_seq
+    kc = (torch.randn(npg, G, 64, D, device=dev) * 0.5).to(bf)
+    vc = (torch.randn(npg, G, D, 64, device=dev) * 0.5).to(bf)
+    bt = torch.arange(npg, dtype=torch.int32, device=dev).view(nseq, pages_seq)
+    r1, r2, pb = (torch.full((H,), v, device=dev) for v in (0.7, 0.2, -1.0))
+    out = {}
+    # ---- prompt portions: nb sequences of L tokens, no earlier context
+    T = nb * L
+    q = torch.randn(T, H * D, device=dev).to(bf)
+    gate = torch.randn(T, H * D, device=dev).to(bf)
+    cu = torch.arange(0, T + 1, L, dtype=torch.int32, device=dev)
+    cx = torch.full((nb,), L, dtype=torch.int32, device=dev)
+    pairs = nb * sum(min(i + 1, W) for i in range(L)) * H          # visible (query, key) pairs
+    flops = 4.0 * pairs * D
+    t_sig = _timed(lambda: ops.sigmoid_attention_prefill(q, gate, kc, vc, bt, cu, cx, L, H, G, D, D, D ** -0.5, W, 4,
+                                                         r1, r2, pb), iters)
+    t_soft = _timed(lambda: ops.prefill_attention_paged(q, kc, vc, bt, cu, cx, H, G, D, L, D ** -0.5, window=W, impl=4),
+                    iters)
+    out["prefill"] = {
+        "sigmoid_ms": round(t_sig * 1e3, 3), "softmax_ms": round(t_soft * 1e3, 3),
+        "sigmoid_mfma_frac": round(flops / t_sig / PEAK_BF16, 4), "softmax_mfma_frac": round(flops / t_soft / PEAK_BF16, 4),
+        "sigmoid_transcendental_frac": round(3.0 * pairs / t_sig / PEAK_TRANS, 4),
+        "softmax_transcendental_frac": round(1.0 * pairs / t_soft / PEAK_TRANS, 4)}
+    # ---- decode rows: nd sequences of ctx keys, one query each
+    qd = torch.randn(nd, H * D, device=dev).to(bf)
+    gd = torch.randn(nd, H * D, device=dev).to(bf)
+    seq = torch.arange(nd, dtype=torch.int32, device=dev)
+    pos = torch.full((nd,), ctx - 1, dtype=torch.int32, device=dev)
+    cxd = torch.full((nd,), ctx, dtype=torch.int32, device=dev)
+    ws = ops.DecodeWorkspace(nd, H, G, ctx, dev, None, D=D)
+    vis = min(ctx, W)
+    kv_bytes = nd * G * vis * D * 2 * 2.0
+    t_sigd = _timed(lambda: ops.sigmoid_attention(qd, gd, kc, vc, bt, seq, pos, H, G, D, D, D ** -0.5, W, 4, r1, r2, pb),
+                    iters)
+    t_softd = _timed(lambda: ops.decode_attention(qd, kc, vc, bt, cxd, H, G, ctx, D ** -0.5, ws=ws, window=W), iters)
+    out["decode"] = {"sigmoid_ms": round(t_sigd * 1e3, 4), "softmax_ms": round(t_softd * 1e3, 4),
+                     "sigmoid_hbm_frac": round(kv_bytes / t_sigd / PEAK_HBM, 4),
+                     "softmax_hbm_frac": round(kv_bytes / t_softd / PEAK_HBM, 4)}
+    return out
+
+
+def run(args) -> None:
+    names = [s for s in (args.design_sizes or "s,m,l").split(",") if s]
+    res = {}
+    for n in names:
+        z = SIZES[n]
+        res[n] = {"shape": {k: v for k, v in z.items()}}
+        for kind in ("bidasun", "mistral"):
+            res[n][kind] = engine_rates(kind, z, max(1, args.steps), max(1, args.warmup))
+            torch.cuda.empty_cache()
+        res[n]["attention_kernels"] = kernel_times(z)
+        torch.cuda.empty_cache()
+        print(f"[designs] {n}: {json.dumps(res[n])}", flush=True)
+    line = {"metric": "design_compare", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "dtype": "bf16", "data": "synthetic token ids, random weights", "sizes": res}
+    print(json.dumps(line), flush=True)
+    if args.out:
+        with open(args.out, "w") as f:
+            f.write(json.dumps(line) + "\n")

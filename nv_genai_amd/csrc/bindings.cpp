@@ -1093,6 +1093,40 @@ void sigmoid_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate,
                                      r1.data_ptr<float>(), r2.data_ptr<float>(), pb.data_ptr<float>(), cur_stream(q));
 }
 
+
+// single-token rows on the MFMA kernel (bf16; dk, dv in {32, 64, 128}; at most 16 query heads per
+// KV head): ws is the fp32 partial workspace [T, Hq, parts * 4, dv]
+void sigmoid_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c10::optional<Tensor> gate, Tensor kc,
+                              Tensor vc, Tensor block_tables, Tensor tok_seq, Tensor pos, int64_t Hq, int64_t Hkv,
+                              int64_t dk, int64_t dv, double scale, int64_t window, int64_t keep_first, Tensor r1,
+                              Tensor r2, Tensor pb) {
+  CHECK_BF16(q); CHECK_BF16(out); CHECK_CONTIG(out); CHECK_F32(ws);
+  CHECK_F32(r1); CHECK_F32(r2); CHECK_F32(pb); CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
+  TORCH_CHECK(nga::sigmoid_attention_mfma_supported((int)dk, (int)dv), "sigmoid_attention_decode: dk, dv in {32, 64, 128}");
+  const int64_t T = q.size(0);
+  TORCH_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && Hq / Hkv <= 16, "at most 16 query heads per KV head");
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == Hq * dk && q.stride(0) % 8 == 0 &&
+              (uintptr_t)q.data_ptr() % 16 == 0, "q must be 16-B aligned [T, Hq * dk] rows");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == Hq * dv);
+  TORCH_CHECK(parts >= 1 && parts <= 64 && ws.numel() >= T * Hq * parts * 4 * dv && (uintptr_t)ws.data_ptr() % 16 == 0);
+  TORCH_CHECK(window > 0 && keep_first >= 0 && r1.numel() == Hq && r2.numel() == Hq && pb.numel() == Hq);
+  TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);
+  check_sig_pages(q, kc, vc, Hkv, dk, dv);
+  const uint16_t* gp = nullptr;
+  int64_t gs = 0;
+  if (gate.has_value()) {
+    CHECK_BF16(*gate);
+    TORCH_CHECK(gate->dim() == 2 && gate->size(0) == T && gate->size(1) == Hq * dv && gate->stride(1) == 1);
+    gp = bfp(*gate);
+    gs = gate->stride(0);
+  }
+  nga::launch_sigmoid_decode_mfma(bfp(out), ws.data_ptr<float>(), (int)parts, bfp(q), q.stride(0), gp, gs, bfp(kc),
+                                  bfp(vc), block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
+                                  tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T, (int)Hq, (int)Hkv, (int)dk,
+                                  (int)dv, (float)scale, (int)window, (int)keep_first, r1.data_ptr<float>(),
+                                  r2.data_ptr<float>(), pb.data_ptr<float>(), cur_stream(q));
+}
+
 }  // namespace
 
 
@@ -1154,6 +1188,10 @@ PYBIND11_MODULE(_C, m) {
   m.def("glu_gelu_tanh", checked("glu_gelu_tanh", &glu_gelu_tanh));
   m.def("qk_norm_cache", checked("qk_norm_cache", &qk_norm_cache));
   m.def("sigmoid_attention", checked("sigmoid_attention", &sigmoid_attention));
+  m.def("sigmoid_attention_decode", checked("sigmoid_attention_decode", &sigmoid_attention_decode));
+  m.def("sigmoid_decode_parts", [](int64_t rows, int64_t Hkv, int64_t max_ctx, int64_t window, int64_t keep) {
+    return (int64_t)nga::sigmoid_decode_parts((int)rows, (int)Hkv, (int)max_ctx, (int)window, (int)keep);
+  });
   m.def("sigmoid_attention_prefill", checked("sigmoid_attention_prefill", &sigmoid_attention_prefill));
   m.def("sigmoid_attention_mfma_supported", [](int64_t dk, int64_t dv) { return nga::sigmoid_attention_mfma_supported((int)dk, (int)dv); });
   m.def("silu_mul", checked("silu_mul", &silu_mul));

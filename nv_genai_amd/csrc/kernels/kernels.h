@@ -252,5 +252,12 @@ void launch_sigmoid_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
                                    const int32_t* ctx_lens, int B, int max_q_len, int Hq, int Hkv, int dk, int dv,
                                    float scale, int window, int keep_first, const float* r1, const float* r2,
                                    const float* pb, hipStream_t stream);
+int sigmoid_decode_parts(int rows, int Hkv, int max_ctx, int window, int keep_first);
+void launch_sigmoid_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
+                                const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
+                                const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
+                                const int32_t* pos, int64_t T, int Hq, int Hkv, int dk, int dv, float scale,
+                                int window, int keep_first, const float* r1, const float* r2, const float* pb,
+                                hipStream_t stream);
 
 }  // namespace nga

@@ -317,6 +317,126 @@ bool launch_sig_mfma_dv(const SigMfmaParams& P, int dv, dim3 grid, hipStream_t s
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// MFMA form for single-token rows (bf16): the query "columns" of the 16-wide tiles are the query
+// heads that share one KV head, so a page is read once for the whole group. Workgroup = 4 waves
+// = (token row, KV head, part); every wave walks its own pages of the row's visible list (kept
+// pages, then the window's pages), strided over the 4 * parts waves of the row, with the K and
+// V^T fragments loaded straight from the page into the MFMA A operands (each byte once, no LDS:
+// nothing is shared between waves). Un-normalised weights make partial sums additive: every
+// wave writes its fp32 partial [group, DV] to a workspace slot and sigmoid_decode_reduce sums
+// the slots in a fixed order, applies the output gate and writes bf16.
+template <int DK, int DV>
+__global__ void __launch_bounds__(256) sigmoid_decode_mfma_kernel(
+    float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
+    const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int Hq, int Hkv, float scale, int window,
+    int keep_first, const float* __restrict__ r1, const float* __restrict__ r2, const float* __restrict__ pb) {
+  constexpr int KT = 64;
+  constexpr int DS = DK / 32;
+  constexpr int DT = DV / 16;
+  const int part = blockIdx.x, parts = gridDim.x, kvh = blockIdx.y;
+  const int64_t row = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, h = lane >> 4;
+  const int grp = Hq / Hkv;
+  const int nslots = parts * 4, slot = part * 4 + w;
+  const bool head_ok = col < grp;
+  const int hq = kvh * grp + (head_ok ? col : 0);
+  const int i = pos[row];
+
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4)(0.f);
+  if (i >= 0) {
+    const int32_t* bt = block_tables + (int64_t)tok_seq[row] * max_blocks;
+    bf16x8 qf[DS];
+    {
+      const uint16_t* qp = q + row * q_stride + (int64_t)hq * DK;
+#pragma unroll
+      for (int s2 = 0; s2 < DS; ++s2) qf[s2] = head_ok ? as_bf16x8(load8(qp + 32 * s2 + 8 * h)) : as_bf16x8((u16x8)(0));
+    }
+    const float a1 = r1[hq], a2 = r2[hq], bias = pb[hq];
+    const int lo = max(0, i - window + 1);
+    const int p_lo = lo / KT, p_hi = i / KT;
+    const int first_cnt = min((min(keep_first, lo) + KT - 1) / KT, p_lo);   // kept pages below the window's
+    const int total = first_cnt + p_hi - p_lo + 1;
+    for (int x = slot; x < total; x += nslots) {
+      const int t = x < first_cnt ? x : p_lo + (x - first_cnt);
+      const int64_t blk = bt[t];
+      const uint16_t* kp = kc + (blk * Hkv + kvh) * (int64_t)(KT * DK);
+      const uint16_t* vp = vc + (blk * Hkv + kvh) * (int64_t)(DV * KT);
+      f32x4 sacc[4];
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau) {
+        const int krow = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
+        sacc[tau] = (f32x4)(0.f);
+#pragma unroll
+        for (int s2 = 0; s2 < DS; ++s2)
+          sacc[tau] = mfma16(as_bf16x8(load8(kp + krow * DK + 32 * s2 + 8 * h)), qf[s2], sacc[tau]);
+      }
+      const int kbase = t * KT;
+      bf16x8 pf[2];
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int key = kbase + 32 * (tau >> 1) + 8 * h + 4 * (tau & 1) + rr;
+          const int dist = i - key;
+          const bool ok = dist >= 0 && (dist < window || key < keep_first);
+          const float z = sacc[tau][rr] * scale - a1 * __logf(1.0f + a2 * (float)dist) + bias;
+          const float wv = ok ? __builtin_amdgcn_rcpf(1.0f + __expf(-z)) : 0.f;
+          pf[tau >> 1][4 * (tau & 1) + rr] = (__bf16)wv;
+        }
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          o[dt] = mfma16(as_bf16x8(load8(vp + (16 * dt + col) * KT + 32 * g + 8 * h)), pf[g], o[dt]);
+    }
+  }
+  if (!head_ok) return;
+  float* wp = ws + ((row * Hq + hq) * nslots + slot) * (int64_t)DV;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(wp + 16 * dt + 4 * h) = o[dt];
+}
+
+// out[row, hq*dv + d] = (sum over slots of ws[row, hq, slot, d]) * sigmoid(gate)
+__global__ void __launch_bounds__(256) sigmoid_decode_reduce_kernel(uint16_t* __restrict__ out,
+                                                                    const float* __restrict__ ws,
+                                                                    const uint16_t* __restrict__ gate,
+                                                                    int64_t g_stride, int64_t total, int HD, int dv,
+                                                                    int nslots) {
+  for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = e / HD;
+    const int c = (int)(e - row * HD);
+    const int hq = c / dv, d = c - hq * dv;
+    const float* wp = ws + ((row * (HD / dv) + hq) * nslots) * (int64_t)dv + d;
+    float acc = 0.f;
+    for (int sl = 0; sl < nslots; ++sl) acc += wp[(int64_t)sl * dv];
+    if (gate) acc *= sigmoidf_(bf2f(gate[row * g_stride + c]));
+    out[e] = f2bf(acc);
+  }
+}
+
+template <int DK>
+bool launch_sig_decode_dv(int dv, dim3 grid, hipStream_t stream, float* ws, const uint16_t* q, int64_t q_stride,
+                          const uint16_t* kc, const uint16_t* vc, const int32_t* bt, int max_blocks,
+                          const int32_t* tok_seq, const int32_t* pos, int Hq, int Hkv, float scale, int window,
+                          int keep_first, const float* r1, const float* r2, const float* pb) {
+#define NGA_SIG_DEC(DV_)                                                                                             \
+  sigmoid_decode_mfma_kernel<DK, DV_><<<grid, 256, 0, stream>>>(ws, q, q_stride, kc, vc, bt, max_blocks, tok_seq, pos, \
+                                                                Hq, Hkv, scale, window, keep_first, r1, r2, pb)
+  switch (dv) {
+    case 32: NGA_SIG_DEC(32); return true;
+    case 64: NGA_SIG_DEC(64); return true;
+    case 128: NGA_SIG_DEC(128); return true;
+    default: return false;
+  }
+#undef NGA_SIG_DEC
+}
+
 }  // namespace
 
 void launch_qk_norm_cache(void* proj, int64_t stride, const float* qw, const float* kw, float eps,
@@ -373,6 +493,42 @@ void launch_sigmoid_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_s
   else if (dk == 64) ok = launch_sig_mfma_dv<64>(P, dv, grid, stream);
   else if (dk == 128) ok = launch_sig_mfma_dv<128>(P, dv, grid, stream);
   if (!ok) abort();   // the caller checks sigmoid_attention_mfma_supported
+}
+
+// Parts (workgroups per row and KV head) of the single-token MFMA kernel: enough waves to fill
+// the chip, never more than the pages a row can see. Fixed by sizes the host knows, so a
+// captured step keeps its launch shape.
+int sigmoid_decode_parts(int rows, int Hkv, int max_ctx, int window, int keep_first) {
+  const int64_t span = (int64_t)window + keep_first;
+  const int pages = (int)((span < max_ctx ? span : max_ctx) / 64) + 2;
+  int by_pages = (pages + 3) / 4;
+  int by_fill = (2048 + rows * Hkv * 4 - 1) / (rows * Hkv * 4);
+  int p = by_pages < by_fill ? by_pages : by_fill;
+  return p < 1 ? 1 : (p > 64 ? 64 : p);
+}
+
+// ws: fp32 [T, Hq, parts * 4, dv]
+void launch_sigmoid_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
+                                const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
+                                const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
+                                const int32_t* pos, int64_t T, int Hq, int Hkv, int dk, int dv, float scale,
+                                int window, int keep_first, const float* r1, const float* r2, const float* pb,
+                                hipStream_t stream) {
+  if (T == 0) return;
+  const dim3 grid((unsigned)parts, (unsigned)Hkv, (unsigned)T);
+  bool ok = false;
+#define NGA_SIG_ARGS dv, grid, stream, ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, Hq, Hkv, scale, \
+                     window, keep_first, r1, r2, pb
+  if (dk == 32) ok = launch_sig_decode_dv<32>(NGA_SIG_ARGS);
+  else if (dk == 64) ok = launch_sig_decode_dv<64>(NGA_SIG_ARGS);
+  else if (dk == 128) ok = launch_sig_decode_dv<128>(NGA_SIG_ARGS);
+#undef NGA_SIG_ARGS
+  if (!ok) abort();   // the caller checks sigmoid_attention_mfma_supported
+  const int64_t total = T * Hq * dv;
+  int64_t g = (total + 255) / 256;
+  if (g > 4096) g = 4096;
+  sigmoid_decode_reduce_kernel<<<dim3((unsigned)g), 256, 0, stream>>>(out, ws, gate, g_stride, total, Hq * dv, dv,
+                                                                     parts * 4);
 }
 
 }  // namespace nga

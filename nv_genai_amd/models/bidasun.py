@@ -59,7 +59,7 @@ class BidasunModel:
         self.k_cache: List[torch.Tensor] = []
         self.v_cache: List[torch.Tensor] = []
         self.shift_state: List[torch.Tensor] = []
-        self.mfma_prefill = True   # prompt portions on the MFMA kernel where it applies (bf16, dims 32 / 64 / 128)
+        self.mfma_prefill = True   # MFMA attention kernels where they apply (bf16, head sizes 32 / 64 / 128)
         if weights is None:
             weights = random_weights(cfg, seed, dtype)
         self._load(weights)
@@ -176,11 +176,14 @@ class BidasunModel:
             # n_decode rows) on the row kernel, into disjoint rows of one output
             a = torch.empty(proj.shape[0], L["ng"], dtype=proj.dtype, device=proj.device)
             if nd:
-                ops.sigmoid_attention(q[:nd], gate[:nd], kc, vc, meta.block_tables, meta.tok_seq[:nd], pos[:nd], *args,
-                                      out=a[:nd])
+                ops.sigmoid_attention_rows(q[:nd], gate[:nd], kc, vc, meta.block_tables, meta.tok_seq[:nd], pos[:nd],
+                                           *args, max_ctx=meta.max_ctx, out=a[:nd])
             ops.sigmoid_attention_prefill(q[nd:], gate[nd:], kc, vc, meta.block_tables[nd:],
                                           meta.cu_q_prefill if nd else meta.cu_q, meta.ctx_lens[nd:],
                                           meta.max_q_len, *args, out=a[nd:])
+        elif meta.kind == "decode" and self.mfma_prefill:
+            a = ops.sigmoid_attention_rows(q, gate, kc, vc, meta.block_tables, meta.tok_seq, pos, *args,
+                                           max_ctx=meta.max_ctx)
         else:
             a = ops.sigmoid_attention(q, gate, kc, vc, meta.block_tables, meta.tok_seq, pos, *args)
         return ops.linear(a, L["wo"])

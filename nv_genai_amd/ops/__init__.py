@@ -435,6 +435,26 @@ def sigmoid_attention_prefill(q, gate, kc, vc, block_tables, cu_q, ctx_lens, max
     return out
 
 
+def sigmoid_attention_rows(q, gate, kc, vc, block_tables, tok_seq, pos, Hq: int, Hkv: int, dk: int, dv: int,
+                           scale: float, window: int, keep_first: int, r1, r2, pb, max_ctx: int, out=None):
+    """:func:`sigmoid_attention` of single-token rows (decode rows; any rows work). bf16 GPU rows
+    with MFMA head sizes and at most 16 query heads per KV head run the page-parallel MFMA kernel
+    (each page read once for the whole head group, fp32 partials summed in a fixed order);
+    everything else takes the row kernel. ``max_ctx`` bounds the rows' positions (launch shape)."""
+    if not (sigmoid_attention_mfma_ok(q, dk, dv) and Hq // Hkv <= 16):
+        return sigmoid_attention(q, gate, kc, vc, block_tables, tok_seq, pos, Hq, Hkv, dk, dv, scale, window,
+                                 keep_first, r1, r2, pb, out=out)
+    C = kernels()
+    T = q.shape[0]
+    parts = C.sigmoid_decode_parts(max(T, 1), Hkv, int(max_ctx), int(window), int(keep_first))
+    ws = torch.empty(T * Hq * parts * 4 * dv, dtype=torch.float32, device=q.device)
+    if out is None:
+        out = torch.empty(T, Hq * dv, dtype=q.dtype, device=q.device)
+    C.sigmoid_attention_decode(out, ws, parts, q, gate, kc, vc, block_tables, tok_seq, pos, Hq, Hkv, dk, dv,
+                               float(scale), int(window), int(keep_first), r1, r2, pb)
+    return out
+
+
 class DecodeWorkspace:
     """Split-K partition buffers for decode attention, sized for (max_seqs, Hq, max_ctx).
 

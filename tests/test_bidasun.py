@@ -220,6 +220,9 @@ def test_one_key_stands_out(device, dtype):
                 qr = q.reshape(T, -1)[rows].contiguous().to(tdt).to(device)
                 tail = (Hq, G, dk, dv, 1.0, W, keep, r1.to(device), r2.to(device), pb.to(device))
                 got = ops.sigmoid_attention(qr, None, kc, vc, bt, seq, pos, *tail)
+                got3 = ops.sigmoid_attention_rows(qr, None, kc, vc, bt, seq, pos, *tail, max_ctx=256)
+                err3 = (got3[-1].double().cpu() - want).abs().max().item()
+                assert err3 < 1e-2, f"single-token kernel: query {i}, key {j}, visible {vis}: off by {err3}"
                 if len(rows) > 1:   # the portion through the prompt kernel too (MFMA tiles in bf16 on the GPU)
                     cu = torch.tensor([0, len(rows)], dtype=torch.int32, device=device)
                     cx = torch.tensor([i + 1], dtype=torch.int32, device=device)
@@ -261,6 +264,15 @@ def test_sigmoid_attention_prompt_portions(device, dtype):
                                             torch.tensor(ctxs, dtype=torch.int32, device=device), 150, Hq, G, dk, dv,
                                             0.2, W, keep, r1.to(device), r2.to(device), pb.to(device))
         close(got, torch.cat(wants), dtype, f"prompt portions {Hq},{G},{dk},{dv},{W},{keep}")
+        # the same rows as single-token rows of a batch (page-parallel MFMA kernel for bf16 on the GPU)
+        seq = torch.tensor([0] * 150 + [1] * 67 + [2] * 2, dtype=torch.int32, device=device)
+        pos = torch.cat([torch.arange(c - n, c) for c, n in zip(ctxs, qlens)]).int().to(device)
+        pick = torch.tensor([0, 13, 149, 150, 216, 217, 218, 77], device=device)
+        got1 = ops.sigmoid_attention_rows(torch.cat(qs).to(device)[pick].contiguous(), torch.cat(gs).to(device)[pick].contiguous(),
+                                          kc, vc, torch.tensor(bts, dtype=torch.int32, device=device),
+                                          seq[pick].contiguous(), pos[pick].contiguous(), Hq, G, dk, dv, 0.2, W, keep,
+                                          r1.to(device), r2.to(device), pb.to(device), max_ctx=256)
+        close(got1, torch.cat(wants)[pick.cpu()], dtype, "single-token rows")
 
 
 # ---------------------------------------------------------------------------- the model on the engine
