@@ -133,8 +133,8 @@ def kernel_times(z: dict, iters: int = 20) -> dict:
     ws = ops.DecodeWorkspace(nd, H, G, ctx, dev, None, D=D)
     vis = min(ctx, W)
     kv_bytes = nd * G * vis * D * 2 * 2.0
-    t_sigd = _timed(lambda: ops.sigmoid_attention(qd, gd, kc, vc, bt, seq, pos, H, G, D, D, D ** -0.5, W, 4, r1, r2, pb),
-                    iters)
+    t_sigd = _timed(lambda: ops.sigmoid_attention_rows(qd, gd, kc, vc, bt, seq, pos, H, G, D, D, D ** -0.5, W, 4, r1, r2,
+                                                       pb, max_ctx=ctx), iters)
     t_softd = _timed(lambda: ops.decode_attention(qd, kc, vc, bt, cxd, H, G, ctx, D ** -0.5, ws=ws, window=W), iters)
     out["decode"] = {"sigmoid_ms": round(t_sigd * 1e3, 4), "softmax_ms": round(t_softd * 1e3, 4),
                      "sigmoid_hbm_frac": round(kv_bytes / t_sigd / PEAK_HBM, 4),

@@ -219,7 +219,13 @@ __global__ void __launch_bounds__(256) sigmoid_attention_mfma_kernel(const SigMf
   const int lo_min = max(0, qpos_lo - W + 1);
   const int t_first = lo_min / KT, t_last = qpos_hi / KT;
   const int t_keep_end = (min(keep, lo_min) + KT - 1) / KT;
-  const float a1 = P.r1[hq], a2 = P.r2[hq], bias = P.pb[hq];
+  const float a1 = P.r1[hq], a2 = P.r2[hq];
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float c0 = -P.scale * LOG2E, c1 = -P.pb[hq] * LOG2E;
+  const float fW = (float)W, fkeep = (float)(qpos - keep);   // key < keep  <=>  distance > qpos - keep
+  // positions of this wave's first and last valid rows
+  const int wq_lo = ctx - qlen + min(qlen - 1, tile * 64 + w * 16);
+  const int wq_hi = ctx - qlen + min(qlen - 1, tile * 64 + w * 16 + 15);
 
   f32x4 o[DT];
 #pragma unroll
@@ -264,17 +270,23 @@ __global__ void __launch_bounds__(256) sigmoid_attention_mfma_kernel(const SigMf
         sacc[tau] = mfma16(a, qf[s2], sacc[tau]);
       }
     }
+    // weights in the exp2 / log2 domain with the constants folded: sigmoid(z) = 1 / (1 + 2^(-z log2e)),
+    // -z log2e = s * c0 + r1 * log2(1 + r2 d) + c1. Distances as floats (exact below 2^24). The
+    // mask costs three compares and a select per score and is only applied on pages that cross
+    // this wave's diagonal, its window's far edge or the end of the kept prefix (wave-uniform).
     const int kbase = t * KT;
+    const float fd = (float)(qpos - kbase - 8 * h);
+    const bool need_mask = kbase + KT - 1 > wq_lo || (wq_hi - kbase >= W && kbase + KT > keep);
     bf16x8 pf[2];
 #pragma unroll
     for (int tau = 0; tau < 4; ++tau)
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        const int key = kbase + 32 * (tau >> 1) + 8 * h + 4 * (tau & 1) + rr;
-        const int dist = qpos - key;
-        const bool ok = dist >= 0 && (dist < W || key < keep);
-        const float z = sacc[tau][rr] * P.scale - a1 * __logf(1.0f + a2 * (float)dist) + bias;
-        const float wv = ok ? __builtin_amdgcn_rcpf(1.0f + __expf(-z)) : 0.f;
+        const float d = fd - (float)(32 * (tau >> 1) + 4 * (tau & 1) + rr);
+        const float lg = __builtin_amdgcn_logf(__builtin_fmaf(a2, d, 1.0f));
+        const float zp = __builtin_fmaf(sacc[tau][rr], c0, __builtin_fmaf(a1, lg, c1));
+        float wv = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zp));
+        if (need_mask) wv = (d >= 0.f && (d < fW || d > fkeep)) ? wv : 0.f;
         pf[tau >> 1][4 * (tau & 1) + rr] = (__bf16)wv;
       }
 #pragma unroll

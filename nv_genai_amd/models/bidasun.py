@@ -59,6 +59,7 @@ class BidasunModel:
         self.k_cache: List[torch.Tensor] = []
         self.v_cache: List[torch.Tensor] = []
         self.shift_state: List[torch.Tensor] = []
+        self.skinny = (self.device.type == "cuda" and dtype == torch.bfloat16 and ops.skinny.enabled())
         self.mfma_prefill = True   # MFMA attention kernels where they apply (bf16, head sizes 32 / 64 / 128)
         if weights is None:
             weights = random_weights(cfg, seed, dtype)
@@ -160,11 +161,23 @@ class BidasunModel:
         raise NotImplementedError("FP8 projections cover the Llama-layout decoders")
 
     # ------------------------------------------------------------------ forward
+    def _lin(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """x @ w^T: decode-shape rows take the skinny MFMA GEMM where the measured table
+        (ops.skinny) holds this (N, K) and prefers it over the library GEMM."""
+        if self.skinny and x.shape[0] <= 512 and x.stride(1) == 1 and x.stride(0) % 8 == 0:
+            pk = ops.skinny.table().pick(w.shape[0], w.shape[1], x.shape[0])
+            if pk is not None:
+                cfg, split = pk
+                if split == 1:
+                    return ops.skinny_gemm(x, w, cfg, 1, 0)
+                return ops.PartialSum(ops.skinny_gemm(x, w, cfg, split, 1)).materialize()
+        return ops.linear(x, w)
+
     def _mixer(self, li: int, h, pos, meta: AttnMeta):
         L = self.layers[li]
         m = L["spec"]
         nq, nk, nv = L["nq"], L["nk"], L["nv"]
-        proj = ops.linear(h, L["wqkvg"])
+        proj = self._lin(h, L["wqkvg"])
         ops.qk_norm_cache_(proj, L["qn"], L["kn"], self.cfg.eps, meta.slots, self.k_cache[li], self.v_cache[li],
                            m.heads, m.kv_heads, m.dim, m.vdim)
         q, gate = proj[:, :nq], proj[:, nq + nk + nv:]
@@ -186,7 +199,7 @@ class BidasunModel:
                                            max_ctx=meta.max_ctx)
         else:
             a = ops.sigmoid_attention(q, gate, kc, vc, meta.block_tables, meta.tok_seq, pos, *args)
-        return ops.linear(a, L["wo"])
+        return self._lin(a, L["wo"])
 
     def forward(self, ids: torch.Tensor, pos: torch.Tensor, meta: AttnMeta,
                 sample_idx: Optional[torch.Tensor] = None, embed_override=None,
@@ -207,7 +220,7 @@ class BidasunModel:
             if "wgu" in L:
                 xb = torch.empty(T, H, dtype=self.dtype, device=x.device)
                 ops.rmsnorm_residual_(x, o, L["norm1"], eps, cast_out=xb)
-                d = ops.linear(ops.glu_gelu_tanh(ops.linear(xb, L["wgu"])), L["wd"])
+                d = self._lin(ops.glu_gelu_tanh(self._lin(xb, L["wgu"])), L["wd"])
                 ops.rmsnorm_residual_(x, d, L["norm2"], eps)
             else:
                 ops.rmsnorm_residual_(x, o, L["norm1"], eps)

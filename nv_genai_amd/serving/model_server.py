@@ -494,7 +494,10 @@ def create_app(llm_service=None, embed_engine=None, rerank_engine=None, llm_name
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("--llm", default="llama3-8b", help="LLM preset ('' to disable)")
+    ap.add_argument("--llm", default="llama3-8b",
+                    help="LLM preset, or a model folder (config.json + safetensors: the design named there, "
+                         "e.g. Bidasun, picks the model class); '' to disable")
+    ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"), help="LLM dtype")
     ap.add_argument("--embed", default="arctic-embed-l", help="encoder preset ('' to disable)")
     ap.add_argument("--rerank", default="", help="reranker preset ('' to disable)")
     ap.add_argument("--vlm", default="", help="vision-language preset, e.g. neva-22b ('' to disable)")
@@ -531,7 +534,8 @@ def main(argv=None):
             from ..utils.checkpoint import load_weights
 
             weights = load_weights(args.weights)
-        eng = LLMEngine(EngineConfig(model=args.llm, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
+        eng = LLMEngine(EngineConfig(model=args.llm, dtype=args.dtype, max_num_seqs=args.max_num_seqs,
+                                     max_model_len=args.max_model_len,
                                      kv_cache_fraction=args.kv_cache_fraction,
                                      kv_cache_dtype=args.kv_cache_dtype, fp8=args.fp8),
                         device=args.device, weights=weights)
