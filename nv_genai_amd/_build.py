@@ -166,9 +166,21 @@ def check_loadable() -> None:
         raise RuntimeError("built extensions do not load:\n" + r.stderr[-2000:])
 
 
-def build_all(force: bool = False) -> None:
-    build_runtime(force=force)
-    build_kernels(force=force)
+def default_jobs() -> int:
+    """Parallel compile jobs: MAX_JOBS when set, else the CPUs this process may use, at most 16."""
+    try:
+        n = int(os.environ.get("MAX_JOBS", "0"))
+    except ValueError:
+        n = 0
+    if n <= 0:
+        n = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 8)
+    return max(1, min(16, n))
+
+
+def build_all(force: bool = False, jobs: int | None = None) -> None:
+    jobs = jobs or default_jobs()
+    build_runtime(force=force, jobs=jobs)
+    build_kernels(force=force, jobs=jobs)
     check_loadable()
 
 
