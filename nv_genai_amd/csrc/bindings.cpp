@@ -1038,8 +1038,8 @@ void sigmoid_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor 
   const int64_t T = q.size(0);
   TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == Hq * dk, "q must be [T, Hq * dk] rows");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == Hq * dv);
-  TORCH_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && dk > 0 && dk <= 1024 && dv > 0 && dv <= 256,
-              "sigmoid_attention: dk <= 1024, dv <= 256");
+  TORCH_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && dk > 0 && dk <= 1024 && dv > 0 && dv <= 512,
+              "sigmoid_attention: dk <= 1024, dv <= 512");
   TORCH_CHECK(window > 0 && keep_first >= 0);
   TORCH_CHECK(r1.numel() == Hq && r2.numel() == Hq && pb.numel() == Hq);
   TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);

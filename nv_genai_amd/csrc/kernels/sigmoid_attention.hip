@@ -76,6 +76,75 @@ __global__ void __launch_bounds__(256) qk_norm_cache_kernel(T* __restrict__ proj
   }
 }
 
+// bf16 rows whose q and k chunks are 16-byte vectors (dk % 8 == 0, nq <= 8192, nk <= 4096): the
+// row stays in registers between the two statistics and the write, so it is read once.
+__global__ void __launch_bounds__(256) qk_norm_cache_vec_kernel(uint16_t* __restrict__ proj, int64_t stride,
+                                                                const float* __restrict__ qw,
+                                                                const float* __restrict__ kw, float eps,
+                                                                const int32_t* __restrict__ slots,
+                                                                uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
+                                                                int Hq, int Hkv, int dk, int dv) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  uint16_t* pr = proj + row * stride;
+  const int nq = Hq * dk, nk = Hkv * dk, nv = Hkv * dv;
+  const int nq8 = nq / 8, nk8 = nk / 8;
+  constexpr int MQ = 4, MK = 2;
+  u16x8 qv[MQ], kv[MK];
+  float sq = 0.f, sk = 0.f;
+#pragma unroll
+  for (int i = 0; i < MQ; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nq8) {
+      qv[i] = load8(pr + c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sq += bf2f(qv[i][j]) * bf2f(qv[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MK; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nk8) {
+      kv[i] = load8(pr + nq + c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sk += bf2f(kv[i][j]) * bf2f(kv[i][j]);
+    }
+  }
+  sq = block_sum(sq, red);
+  sk = block_sum(sk, red);
+  const float rq = 1.0f / sqrtf(sq / (float)nq + eps);
+  const float rk = 1.0f / sqrtf(sk / (float)nk + eps);
+#pragma unroll
+  for (int i = 0; i < MQ; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nq8) {
+      u16x8 o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = f2bf(bf2f(qv[i][j]) * rq * qw[c * 8 + j]);
+      store8(pr + c * 8, o);
+    }
+  }
+  const int slot = slots[row];
+  if (slot < 0) return;
+  const int64_t page = slot / BS;
+  const int off = slot % BS;
+#pragma unroll
+  for (int i = 0; i < MK; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nk8) {
+      const int e = c * 8, hh = e / dk, d = e - hh * dk;
+      u16x8 o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = f2bf(bf2f(kv[i][j]) * rk * kw[e + j]);
+      store8(kc + ((page * Hkv + hh) * BS + off) * dk + d, o);
+    }
+  }
+  for (int c = threadIdx.x; c < nv; c += blockDim.x) {
+    const int hh = c / dv, d = c - hh * dv;
+    vc[((page * Hkv + hh) * dv + d) * BS + off] = pr[nq + nk + c];
+  }
+}
+
 // One wave per (token row, head). q: row stride q_stride, head h at h*dk. gate: row stride
 // g_stride, head h at h*dv (nullptr: no gate). out [T, Hq*dv].
 template <typename T>
@@ -102,8 +171,8 @@ __global__ void __launch_bounds__(64) sigmoid_attention_kernel(
   const int32_t* bt = block_tables + (int64_t)seq * max_blocks;
   for (int d = lane; d < dk; d += 64) qs[d] = ldf(q + row * q_stride + (int64_t)h * dk + d);
   const float a1 = r1[h], a2 = r2[h], b = pb[h];
-  constexpr int MAXV = 4;   // dv <= 256
-  float acc[MAXV] = {0.f, 0.f, 0.f, 0.f};
+  constexpr int MAXV = 8;   // dv <= 512
+  float acc[MAXV] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int lo = i - window + 1 > 0 ? i - window + 1 : 0;   // first key inside the window
   const int keep = keep_first < lo ? keep_first : lo;        // kept keys [0, keep) below the window
   const int p_keep_end = (keep + BS - 1) / BS;               // pages [0, p_keep_end) hold kept keys
@@ -458,6 +527,10 @@ void launch_qk_norm_cache(void* proj, int64_t stride, const float* qw, const flo
   if (f32)
     qk_norm_cache_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>((float*)proj, stride, qw, kw, eps, slots,
                                                                       (float*)kc, (float*)vc, Hq, Hkv, dk, dv);
+  else if (dk % 8 == 0 && stride % 8 == 0 && Hq * dk <= 8192 && Hkv * dk <= 4096 &&
+           ((uintptr_t)proj | (uintptr_t)kc) % 16 == 0)
+    qk_norm_cache_vec_kernel<<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)proj, stride, qw, kw, eps, slots,
+                                                                   (uint16_t*)kc, (uint16_t*)vc, Hq, Hkv, dk, dv);
   else
     qk_norm_cache_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)proj, stride, qw, kw, eps, slots,
                                                                          (uint16_t*)kc, (uint16_t*)vc, Hq, Hkv, dk,

@@ -142,25 +142,27 @@ def _paged(q, k, v, device, tdt, bt_row):
 def test_qk_norm_and_cache_write(device, dtype):
     torch.manual_seed(2)
     tdt = getattr(torch, dtype)
-    Hq, G, dk, dv, T = 4, 2, 8, 12, 70
-    nq, nk, nv = Hq * dk, G * dk, G * dv
-    proj = torch.randn(T, nq + nk + nv + 5).to(tdt)
-    qw, kw = torch.rand(nq) + 0.5, torch.rand(nk) + 0.5
-    bt = [5, 2]
-    slots = torch.tensor([bt[t // 64] * 64 + t % 64 for t in range(T)], dtype=torch.int32)
-    slots[3] = -1                                       # a row that writes nothing
-    kc = torch.zeros(6, G, 64, dk, dtype=tdt, device=device)
-    vc = torch.zeros(6, G, dv, 64, dtype=tdt, device=device)
-    p64 = proj.double()
-    pd = proj.clone().to(device)
-    ops.qk_norm_cache_(pd, qw.to(device), kw.to(device), 1e-5, slots.to(device), kc, vc, Hq, G, dk, dv)
-    close(pd[:, :nq], O.o_rms(p64[:, :nq], qw.double(), 1e-5), dtype, "q norm over the whole projection")
-    kn = O.o_rms(p64[:, nq:nq + nk], kw.double(), 1e-5).view(T, G, dk)
-    for t in (0, 63, 64, 69):
-        close(kc[bt[t // 64], :, t % 64, :], kn[t], dtype, f"k page row {t}")
-        close(vc[bt[t // 64], :, :, t % 64], p64[t, nq + nk:nq + nk + nv].view(G, dv), dtype, f"v page row {t}")
-    assert kc[bt[0], :, 3].abs().sum() == 0
-    close(pd[:, nq + nk:], p64[:, nq + nk:], dtype, "v and the rest untouched")
+    # (heads, kv heads, dim, vdim, extra columns): unaligned rows, and 16-byte-aligned ones (vector kernel)
+    for Hq, G, dk, dv, pad in ((4, 2, 8, 12, 5), (4, 2, 16, 8, 64), (40, 8, 128, 32, 0)):
+        T = 70
+        nq, nk, nv = Hq * dk, G * dk, G * dv
+        proj = torch.randn(T, nq + nk + nv + pad).to(tdt)
+        qw, kw = torch.rand(nq) + 0.5, torch.rand(nk) + 0.5
+        bt = [5, 2]
+        slots = torch.tensor([bt[t // 64] * 64 + t % 64 for t in range(T)], dtype=torch.int32)
+        slots[3] = -1                                       # a row that writes nothing
+        kc = torch.zeros(6, G, 64, dk, dtype=tdt, device=device)
+        vc = torch.zeros(6, G, dv, 64, dtype=tdt, device=device)
+        p64 = proj.double()
+        pd = proj.clone().to(device)
+        ops.qk_norm_cache_(pd, qw.to(device), kw.to(device), 1e-5, slots.to(device), kc, vc, Hq, G, dk, dv)
+        close(pd[:, :nq], O.o_rms(p64[:, :nq], qw.double(), 1e-5), dtype, "q norm over the whole projection")
+        kn = O.o_rms(p64[:, nq:nq + nk], kw.double(), 1e-5).view(T, G, dk)
+        for t in (0, 63, 64, 69):
+            close(kc[bt[t // 64], :, t % 64, :], kn[t], dtype, f"k page row {t}")
+            close(vc[bt[t // 64], :, :, t % 64], p64[t, nq + nk:nq + nk + nv].view(G, dv), dtype, f"v page row {t}")
+        assert kc[bt[0], :, 3].abs().sum() == 0
+        close(pd[:, nq + nk:], p64[:, nq + nk:], dtype, "v and the rest untouched")
 
 
 @pytest.mark.parametrize("device,dtype", DTYPES)
@@ -378,6 +380,21 @@ def test_pipelined_generation_matches_synchronous(device):
     prompts = [tokens(40, seed=31), tokens(70, seed=32)]
     sp = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
     assert [r.output_ids for r in a.generate(prompts, sp)] == [r.output_ids for r in b.generate(prompts, sp)]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_preemption_recomputes_state(device):
+    """A pool too small for both sequences to grow: the scheduler preempts one (its pages and its
+    state slot go back), recomputes it later from its first token, and the tokens do not change."""
+    small, cd, W = build(device, "float32", pages=5)
+    big, _, _ = build(device, "float32", pages=16)
+    prompts = [tokens(120, seed=41), tokens(120, seed=42)]
+    sp = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
+    got = [r.output_ids for r in small.generate(prompts, sp)]
+    assert small.sched.preemptions() > 0
+    assert got == [r.output_ids for r in big.generate(prompts, sp)]
+    assert got[0] == O.o_greedy(cd, W, prompts[0], 20)
+    assert small.sched.free_state_slots() == 4 and small.sched.free_blocks() == 5
 
 
 def test_model_folder_roundtrip(tmp_path):
