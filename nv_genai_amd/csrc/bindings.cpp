@@ -981,13 +981,19 @@ void rmsnorm_f32(Tensor out, Tensor x, c10::optional<Tensor> rows, Tensor w, dou
                           (int)x.size(1), f32, cur_stream(x));
 }
 
-void token_shift(Tensor h, Tensor x, Tensor mu, Tensor src, Tensor state) {
+void token_shift(Tensor h, Tensor x, Tensor mu, Tensor src, Tensor state, c10::optional<Tensor> save) {
   CHECK_F32(x); CHECK_F32(mu); CHECK_F32(state); CHECK_I32(src); CHECK_CONTIG(h);
   const bool f32 = act_f32(h);
   TORCH_CHECK(x.dim() == 2 && h.sizes() == x.sizes() && mu.numel() == x.size(1) && src.numel() == x.size(0));
   TORCH_CHECK(state.dim() == 2 && state.size(1) == x.size(1));
+  const int32_t* sp = nullptr;
+  if (save.has_value()) {
+    CHECK_I32(*save);
+    TORCH_CHECK(save->numel() == x.size(0), "token_shift: one save slot per row");
+    sp = save->data_ptr<int32_t>();
+  }
   nga::launch_token_shift(h.data_ptr(), x.data_ptr<float>(), mu.data_ptr<float>(), src.data_ptr<int32_t>(),
-                          state.data_ptr<float>(), x.size(0), (int)x.size(1), f32, cur_stream(x));
+                          state.data_ptr<float>(), sp, x.size(0), (int)x.size(1), f32, cur_stream(x));
 }
 
 void shift_save(Tensor state, Tensor x, Tensor last_row, Tensor slot) {

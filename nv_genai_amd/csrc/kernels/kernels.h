@@ -230,8 +230,8 @@ void launch_rmsnorm_residual(float* x, const void* y, int64_t y_stride, const fl
                              void* cast_out, bool f32, hipStream_t stream);
 void launch_rmsnorm_f32(void* out, const float* x, const int64_t* rows, const float* w, float eps, int64_t T, int H,
                         bool f32, hipStream_t stream);
-void launch_token_shift(void* h, const float* x, const float* mu, const int32_t* src, const float* state, int64_t T,
-                        int H, bool f32, hipStream_t stream);
+void launch_token_shift(void* h, const float* x, const float* mu, const int32_t* src, float* state,
+                        const int32_t* save, int64_t T, int H, bool f32, hipStream_t stream);
 void launch_shift_save(float* state, const float* x, const int32_t* last_row, const int32_t* slot, int n, int H,
                        hipStream_t stream);
 void launch_glu_gelu_tanh(void* out, const void* in, int64_t T, int F, bool f32, hipStream_t stream);

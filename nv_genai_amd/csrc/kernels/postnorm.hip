@@ -72,18 +72,24 @@ __global__ void __launch_bounds__(256) rmsnorm_f32_kernel(T* __restrict__ out, c
   for (int c = threadIdx.x; c < H; c += blockDim.x) stf(out + (int64_t)blockIdx.x * H + c, xr[c] * r * w[c]);
 }
 
-// src[t] >= 0: row of x; -1: zeros; <= -2: state slot -(src + 2)
+// src[t] >= 0: row of x; -1: zeros; <= -2: state slot -(src + 2). save (optional, one entry per
+// row): slot that takes this row's x afterwards. Only valid when every row is the single token of
+// its sequence (then the row that reads a slot is the row that writes it, element by element in
+// one thread); steps with longer portions save with shift_save after this kernel.
 template <typename T>
 __global__ void __launch_bounds__(256) token_shift_kernel(T* __restrict__ h, const float* __restrict__ x,
                                                           const float* __restrict__ mu, const int32_t* __restrict__ src,
-                                                          const float* __restrict__ state, int H) {
+                                                          float* __restrict__ state, const int32_t* __restrict__ save,
+                                                          int H) {
   const int64_t row = blockIdx.x;
   const int s = src[row];
   const float* prev = s >= 0 ? x + (int64_t)s * H : (s == -1 ? nullptr : state + (int64_t)(-(s + 2)) * H);
+  const int sv = save ? save[row] : -1;
   for (int c = threadIdx.x; c < H; c += blockDim.x) {
     const float v = x[row * H + c];
     const float p = prev ? prev[c] : 0.f;
     stf(h + row * H + c, v + (p - v) * mu[c]);
+    if (sv >= 0) state[(int64_t)sv * H + c] = v;
   }
 }
 
@@ -143,13 +149,13 @@ void launch_rmsnorm_f32(void* out, const float* x, const int64_t* rows, const fl
     rmsnorm_f32_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)out, x, rows, w, eps, H);
 }
 
-void launch_token_shift(void* h, const float* x, const float* mu, const int32_t* src, const float* state, int64_t T,
-                        int H, bool f32, hipStream_t stream) {
+void launch_token_shift(void* h, const float* x, const float* mu, const int32_t* src, float* state,
+                        const int32_t* save, int64_t T, int H, bool f32, hipStream_t stream) {
   if (T == 0) return;
   if (f32)
-    token_shift_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>((float*)h, x, mu, src, state, H);
+    token_shift_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>((float*)h, x, mu, src, state, save, H);
   else
-    token_shift_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)h, x, mu, src, state, H);
+    token_shift_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>((uint16_t*)h, x, mu, src, state, save, H);
 }
 
 void launch_shift_save(float* state, const float* x, const int32_t* last_row, const int32_t* slot, int n, int H,

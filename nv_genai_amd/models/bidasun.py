@@ -214,8 +214,12 @@ class BidasunModel:
         x = ops.embed_pos(ids, pos, self.embed, self.pos_table)
         T, H = x.shape
         for li, L in enumerate(self.layers):
-            h = ops.token_shift(x, L["shift"], meta.shift_src, self.shift_state[li], self.dtype)
-            ops.shift_save_(self.shift_state[li], x, meta.state_rows, meta.state_slots)
+            if meta.kind == "decode":   # one token per sequence: the shift kernel also leaves x in the slot
+                h = ops.token_shift(x, L["shift"], meta.shift_src, self.shift_state[li], self.dtype,
+                                    save_slots=meta.state_slots)
+            else:
+                h = ops.token_shift(x, L["shift"], meta.shift_src, self.shift_state[li], self.dtype)
+                ops.shift_save_(self.shift_state[li], x, meta.state_rows, meta.state_slots)
             o = self._mixer(li, h, pos, meta)
             if "wgu" in L:
                 xb = torch.empty(T, H, dtype=self.dtype, device=x.device)

@@ -343,14 +343,21 @@ def rmsnorm_f32(x: torch.Tensor, w: torch.Tensor, eps: float, rows: Optional[tor
 
 
 def token_shift(x: torch.Tensor, mu: torch.Tensor, src: torch.Tensor, state: torch.Tensor,
-                dtype: torch.dtype) -> torch.Tensor:
+                dtype: torch.dtype, save_slots: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Token shift: ``h[t] = x[t] + (prev(t) - x[t]) * mu`` with prev(t) the input one token
     earlier. ``src[t]`` says where it is: >= 0 a row of ``x`` (same step), -1 zeros (first token
-    of a sequence), <= -2 row ``-(src + 2)`` of ``state`` [slots, H] (the step before)."""
+    of a sequence), <= -2 row ``-(src + 2)`` of ``state`` [slots, H] (the step before).
+    ``save_slots`` (one per row, negative: none): also store ``x[t]`` into that state slot, in the
+    same launch. Only for steps whose rows are each the single token of their sequence (decode
+    steps): there the row that reads a slot is the one that writes it. Other steps call
+    :func:`shift_save_` afterwards."""
     if not _gpu(x):
-        return ref.token_shift(x, mu, src, state, dtype)
+        h = ref.token_shift(x, mu, src, state, dtype)
+        if save_slots is not None:
+            ref.shift_save_(state, x, torch.arange(x.shape[0], dtype=torch.int32), save_slots)
+        return h
     h = torch.empty(x.shape, dtype=dtype, device=x.device)
-    kernels().token_shift(h, x, mu, src, state)
+    kernels().token_shift(h, x, mu, src, state, save_slots)
     return h
 
 

@@ -108,6 +108,17 @@ def test_token_shift_and_state(device):
     h2 = ops.token_shift(xd[5:].contiguous(), mud, src2, state, torch.float32)
     close(torch.cat([h1, h2]), want, "float32", "token shift")
     assert state[0].abs().sum() == 0 and state[1].abs().sum() == 0
+    # decode rows: two sequences, one token each per step; the shift itself leaves x in the slots
+    y = torch.randn(4, 2, 20)                            # [step, sequence, width]
+    st = torch.zeros(3, 20, device=device)
+    slots = torch.tensor([2, 0], dtype=torch.int32, device=device)
+    outs = []
+    for t in range(4):
+        src = torch.tensor([-1, -1] if t == 0 else [-4, -2], dtype=torch.int32, device=device)
+        outs.append(ops.token_shift(y[t].to(device).contiguous(), mud, src, st, torch.float32, save_slots=slots))
+    for b in range(2):
+        close(torch.stack([o[b] for o in outs]), O.o_token_shift(y[:, b].double(), mu.double()), "float32", "decode rows")
+    assert st[1].abs().sum() == 0
 
 
 @pytest.mark.parametrize("device,dtype", DTYPES)
