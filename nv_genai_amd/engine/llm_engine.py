@@ -1162,7 +1162,7 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
             for rid, toks, _ in rows:
                 toks = [int(t) for t in toks]
                 if not toks:
-                    raise ValueError("a replayed row needs at least one token")
+                    continue   # a row that brings nothing this step
                 if rid in live:
                     self.sched.extend(rid, toks)
                 else:
@@ -1182,7 +1182,7 @@ class LLMEngine(ReplicaMixin, StepGraphMixin):
                 row_of = {int(x): i for i, x in enumerate(sid[:n].tolist())}
                 want = [int(cu[row_of[int(rid)]]) + int(w) for rid, toks, ws in rows for w in ws
                         if 0 <= int(w) < len(toks)]
-                if sum(len(ws) for _, _, ws in rows) != len(want):
+                if sum(len(ws) for _, toks, ws in rows if len(toks)) != len(want):
                     raise ValueError("a wanted place lies outside its row's tokens")
                 self._count(kind, n, ntok, nd)
                 logits = self._replay_forward(kind, n, ntok, nd, want, layer_tap)
