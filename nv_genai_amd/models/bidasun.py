@@ -20,7 +20,6 @@ scheduler assigns. The serving engine drives this class exactly as it drives
 """
 from __future__ import annotations
 
-import math
 from typing import Dict, List, Optional
 
 import torch

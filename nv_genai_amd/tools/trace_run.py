@@ -49,7 +49,6 @@ def main(argv=None) -> int:
     a = ap.parse_args(argv)
     if a.device.startswith("cuda"):
         _ensure_built()
-    import numpy as np
     import torch
 
     from ..engine.llm_engine import EngineConfig, LLMEngine

@@ -5,8 +5,6 @@ state slots, row maps) and, marked ``gpu``, on the HIP kernels in float32 and bf
 models are small random ones built here; their sizes are chosen so that no two of heads,
 kv heads, dim, vdim, window, keep_first and the page size coincide.
 """
-import math
-
 import pytest
 import torch
 
