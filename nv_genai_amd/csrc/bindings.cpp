@@ -1101,7 +1101,7 @@ void sigmoid_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate,
 
 
 // single-token rows on the MFMA kernel (bf16; dk, dv in {32, 64, 128}; at most 16 query heads per
-// KV head): ws is the fp32 partial workspace [T, Hq, parts * 4, dv]
+// KV head): ws is the fp32 partial workspace [T, Hq, parts, dv]
 void sigmoid_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c10::optional<Tensor> gate, Tensor kc,
                               Tensor vc, Tensor block_tables, Tensor tok_seq, Tensor pos, int64_t Hq, int64_t Hkv,
                               int64_t dk, int64_t dv, double scale, int64_t window, int64_t keep_first, Tensor r1,
@@ -1114,7 +1114,7 @@ void sigmoid_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c1
   TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == Hq * dk && q.stride(0) % 8 == 0 &&
               (uintptr_t)q.data_ptr() % 16 == 0, "q must be 16-B aligned [T, Hq * dk] rows");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == Hq * dv);
-  TORCH_CHECK(parts >= 1 && parts <= 64 && ws.numel() >= T * Hq * parts * 4 * dv && (uintptr_t)ws.data_ptr() % 16 == 0);
+  TORCH_CHECK(parts >= 1 && parts <= 64 && ws.numel() >= T * Hq * parts * dv && (uintptr_t)ws.data_ptr() % 16 == 0);
   TORCH_CHECK(window > 0 && keep_first >= 0 && r1.numel() == Hq && r2.numel() == Hq && pb.numel() == Hq);
   TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);
   check_sig_pages(q, kc, vc, Hkv, dk, dv);
@@ -1148,7 +1148,7 @@ const FormSpec kForms[KF_COUNT] = {
     {"decode_dma", "NGA_DECODE_DMA", 2}, {"decode_nt", "NGA_DECODE_NT", 2},
     {"search_dma", "NGA_SEARCH_DMA", 1}, {"prefill_v1", "NGA_PREFILL_V1", 0},
     {"prefill_ks", "NGA_PREFILL_KS", 0}, {"rope_vnt", "NGA_ROPE_VNT", 2},
-    {"decode_dma_aux", "NGA_DECODE_DMA_AUX", 2}};
+    {"decode_dma_aux", "NGA_DECODE_DMA_AUX", 2}, {"sig_decode_waves", "NGA_SIG_DECODE_WAVES", 8192}};
 std::atomic<int>* forms() {
   static std::atomic<int> v[KF_COUNT];
   static const bool init = [] {

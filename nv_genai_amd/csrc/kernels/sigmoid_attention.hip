@@ -405,8 +405,8 @@ bool launch_sig_mfma_dv(const SigMfmaParams& P, int dv, dim3 grid, hipStream_t s
 // pages, then the window's pages), strided over the 4 * parts waves of the row, with the K and
 // V^T fragments loaded straight from the page into the MFMA A operands (each byte once, no LDS:
 // nothing is shared between waves). Un-normalised weights make partial sums additive: every
-// wave writes its fp32 partial [group, DV] to a workspace slot and sigmoid_decode_reduce sums
-// the slots in a fixed order, applies the output gate and writes bf16.
+// workgroup sums its four waves' fp32 partials [group, DV] through LDS into one workspace slot and
+// sigmoid_decode_reduce sums the slots in a fixed order, applies the output gate and writes bf16.
 template <int DK, int DV>
 __global__ void __launch_bounds__(256) sigmoid_decode_mfma_kernel(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
@@ -422,7 +422,7 @@ __global__ void __launch_bounds__(256) sigmoid_decode_mfma_kernel(
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, h = lane >> 4;
   const int grp = Hq / Hkv;
-  const int nslots = parts * 4, slot = part * 4 + w;
+  const int nslots = parts * 4, slot = part * 4 + w;   // the row's pages are strided over all its waves
   const bool head_ok = col < grp;
   const int hq = kvh * grp + (head_ok ? col : 0);
   const int i = pos[row];
@@ -477,10 +477,18 @@ __global__ void __launch_bounds__(256) sigmoid_decode_mfma_kernel(
           o[dt] = mfma16(as_bf16x8(load8(vp + (16 * dt + col) * KT + 32 * g + 8 * h)), pf[g], o[dt]);
     }
   }
-  if (!head_ok) return;
-  float* wp = ws + ((row * Hq + hq) * nslots + slot) * (int64_t)DV;
+  // the workgroup's four partials -> one slot: through LDS, summed in wave order
+  __shared__ float red_s[4][DV][17];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(wp + 16 * dt + 4 * h) = o[dt];
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) red_s[w][16 * dt + 4 * h + rr][col] = o[dt][rr];
+  __syncthreads();
+  for (int e = tid; e < grp * DV; e += 256) {
+    const int c = e / DV, d = e - c * DV;
+    const float sum = ((red_s[0][d][c] + red_s[1][d][c]) + red_s[2][d][c]) + red_s[3][d][c];
+    ws[((row * Hq + kvh * grp + c) * parts + part) * (int64_t)DV + d] = sum;
+  }
 }
 
 // out[row, hq*dv + d] = (sum over slots of ws[row, hq, slot, d]) * sigmoid(gate)
@@ -587,12 +595,14 @@ int sigmoid_decode_parts(int rows, int Hkv, int max_ctx, int window, int keep_fi
   const int64_t span = (int64_t)window + keep_first;
   const int pages = (int)((span < max_ctx ? span : max_ctx) / 64) + 2;
   int by_pages = (pages + 3) / 4;
-  int by_fill = (2048 + rows * Hkv * 4 - 1) / (rows * Hkv * 4);
+  int target = kernel_form(KF_SIG_DECODE_WAVES);   // waves to launch: 8192 = 8 per SIMD on 256 CUs
+  if (target < 1) target = 1;
+  int by_fill = (target + rows * Hkv * 4 - 1) / (rows * Hkv * 4);
   int p = by_pages < by_fill ? by_pages : by_fill;
   return p < 1 ? 1 : (p > 64 ? 64 : p);
 }
 
-// ws: fp32 [T, Hq, parts * 4, dv]
+// ws: fp32 [T, Hq, parts, dv]
 void launch_sigmoid_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
                                 const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
                                 const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
@@ -613,7 +623,7 @@ void launch_sigmoid_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
   int64_t g = (total + 255) / 256;
   if (g > 4096) g = 4096;
   sigmoid_decode_reduce_kernel<<<dim3((unsigned)g), 256, 0, stream>>>(out, ws, gate, g_stride, total, Hq * dv, dv,
-                                                                     parts * 4);
+                                                                     parts);
 }
 
 }  // namespace nga

@@ -454,7 +454,7 @@ def sigmoid_attention_rows(q, gate, kc, vc, block_tables, tok_seq, pos, Hq: int,
     C = kernels()
     T = q.shape[0]
     parts = C.sigmoid_decode_parts(max(T, 1), Hkv, int(max_ctx), int(window), int(keep_first))
-    ws = torch.empty(T * Hq * parts * 4 * dv, dtype=torch.float32, device=q.device)
+    ws = torch.empty(T * Hq * parts * dv, dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty(T, Hq * dv, dtype=q.dtype, device=q.device)
     C.sigmoid_attention_decode(out, ws, parts, q, gate, kc, vc, block_tables, tok_seq, pos, Hq, Hkv, dk, dv,
