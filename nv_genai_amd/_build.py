@@ -97,7 +97,10 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> 
     objdir.mkdir(parents=True, exist_ok=True)
     inc, defs, libs = _torch_flags()
     hip_srcs = sorted((CSRC / "kernels").glob("*.hip"))
-    common = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}", "-Wno-unused-result"]
+    # no packed-fp32 VALU forms (v_pk_*_f32): hipcc -O3 makes them from plain float code, and
+    # some of their forms have given wrong results on this hardware now and then
+    common = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}", "-Wno-unused-result",
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     if os.environ.get("NGA_DIAG_BUILD", "0") != "0":
         # kernel ablation variants (NGA_PV2_ABLATE / NGA_MOE_ABLATE: timings only, results
         # wrong by design) exist only in this build; rebuild with force=True when switching

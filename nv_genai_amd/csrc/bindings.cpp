@@ -1133,6 +1133,164 @@ void sigmoid_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c1
                                   r2.data_ptr<float>(), pb.data_ptr<float>(), cur_stream(q));
 }
 
+// ------------------------------------------------------------------ sandwich norms, head-map softmax attention, recurrence
+void embed_rows(Tensor x, Tensor ids, Tensor embed, double scale) {
+  CHECK_F32(x); CHECK_I32(ids);
+  const bool f32 = act_f32(embed);
+  CHECK_CONTIG(embed);
+  TORCH_CHECK(x.dim() == 2 && embed.dim() == 2 && embed.size(1) == x.size(1) && ids.numel() == x.size(0));
+  nga::launch_embed_rows(x.data_ptr<float>(), ids.data_ptr<int32_t>(), embed.data_ptr(), (float)scale, x.size(0),
+                         (int)x.size(1), (int)embed.size(0), f32, cur_stream(x));
+}
+
+void rmsnorm_residual_next(Tensor x, Tensor y, Tensor w, double eps, Tensor next_w, Tensor out) {
+  CHECK_F32(x); CHECK_F32(w); CHECK_F32(next_w); CHECK_CONTIG(out);
+  const bool f32 = act_f32(y);
+  const int64_t H = x.size(1);
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && y.size(0) == x.size(0) && y.size(1) == H && y.stride(1) == 1);
+  TORCH_CHECK((w.numel() == H || w.numel() == 1) && (next_w.numel() == H || next_w.numel() == 1),
+              "norm weights hold one element or one per coordinate");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == y.scalar_type() && out.sizes() == x.sizes());
+  nga::launch_rmsnorm_residual_next(x.data_ptr<float>(), y.data_ptr(), y.stride(0), w.data_ptr<float>(), (int)w.numel(),
+                                    next_w.data_ptr<float>(), (int)next_w.numel(), (float)eps, x.size(0), (int)H,
+                                    out.data_ptr(), f32, cur_stream(x));
+}
+
+void relu_sq(Tensor out, Tensor x) {
+  const bool f32 = act_f32(x);
+  CHECK_CONTIG(out); CHECK_CONTIG(x);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == x.scalar_type() && out.numel() == x.numel());
+  nga::launch_relu_sq(out.data_ptr(), x.data_ptr(), x.numel(), f32, cur_stream(x));
+}
+
+void softcap(Tensor z, double cap) {
+  CHECK_F32(z);
+  TORCH_CHECK(cap > 0);
+  nga::launch_softcap(z.data_ptr<float>(), z.numel(), (float)cap, cur_stream(z));
+}
+
+void group_rmsnorm(Tensor out, Tensor x, Tensor w, int64_t groups, double eps) {
+  CHECK_F32(x); CHECK_F32(w); CHECK_CONTIG(out);
+  const bool f32 = act_f32(out);
+  TORCH_CHECK(x.dim() == 2 && out.sizes() == x.sizes() && groups > 0 && x.size(1) % groups == 0 &&
+              w.numel() == x.size(1) / groups);
+  nga::launch_group_rmsnorm(out.data_ptr(), x.data_ptr<float>(), w.data_ptr<float>(), x.size(0), (int)groups,
+                            (int)(x.size(1) / groups), (float)eps, f32, cur_stream(x));
+}
+
+// K [blocks, nk, 64, dk] and V [blocks, nv, 64, dv] pages of the activation type
+void check_row_pages(const Tensor& act, const Tensor& c, int64_t heads, int64_t d, const char* what) {
+  TORCH_CHECK(c.is_cuda() && c.is_contiguous() && c.scalar_type() == act.scalar_type(), what,
+              ": pages must be contiguous and of the activation type");
+  TORCH_CHECK(c.dim() == 4 && c.size(1) == heads && c.size(2) == 64 && c.size(3) == d, what,
+              ": pages must be [blocks, heads, 64, d]");
+}
+
+const float* opt_f32(const c10::optional<Tensor>& t, int64_t n, const char* what) {
+  if (!t.has_value()) return nullptr;
+  TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat && t->is_contiguous() && t->numel() == n, what,
+              ": fp32 vector of the wrong size");
+  return t->data_ptr<float>();
+}
+
+void headnorm_cache(Tensor proj, Tensor slots, Tensor kc, c10::optional<Tensor> vc, int64_t nq, int64_t nk, int64_t dk,
+                    int64_t nv, int64_t dv, double eps, c10::optional<Tensor> qw, c10::optional<Tensor> kw,
+                    c10::optional<Tensor> bias, c10::optional<Tensor> pos, double coef, int64_t every) {
+  const bool f32 = act_f32(proj);
+  CHECK_I32(slots);
+  const int64_t n2 = (nq + nk) * dk + nv * dv;
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(1) >= n2 && slots.numel() == proj.size(0));
+  TORCH_CHECK(nq >= 0 && nk >= 0 && nv >= 0 && dk > 0 && every >= 1);
+  if (nk > 0) check_row_pages(proj, kc, nk, dk, "headnorm_cache (k)");
+  void* vp = nullptr;
+  if (nv > 0) {
+    TORCH_CHECK(vc.has_value(), "headnorm_cache: v pages missing");
+    check_row_pages(proj, *vc, nv, dv, "headnorm_cache (v)");
+    TORCH_CHECK(nk == 0 || vc->size(0) == kc.size(0));
+    vp = vc->data_ptr();
+  }
+  const int32_t* pp = nullptr;
+  if (coef != 0.0) {
+    TORCH_CHECK(pos.has_value(), "headnorm_cache: the query temperature needs positions");
+    CHECK_I32(*pos);
+    TORCH_CHECK(pos->numel() == proj.size(0));
+    pp = pos->data_ptr<int32_t>();
+  }
+  nga::launch_headnorm_cache(proj.data_ptr(), proj.stride(0), slots.data_ptr<int32_t>(), nk > 0 ? kc.data_ptr() : nullptr,
+                             vp, proj.size(0), (int)nq, (int)nk, (int)dk, (int)nv, (int)dv, (float)eps,
+                             opt_f32(qw, dk, "q norm weight"), opt_f32(kw, dk, "k norm weight"),
+                             opt_f32(bias, n2, "bias"), pp, (float)coef, (int)every, f32, cur_stream(proj));
+}
+
+struct SoftmaxArgs {
+  const void* gp = nullptr;
+  int64_t gs = 0;
+};
+
+SoftmaxArgs check_softmax_args(const Tensor& out, const Tensor& q, const c10::optional<Tensor>& gate, const Tensor& kc,
+                               const Tensor& vc, int64_t H, int64_t G, int64_t dk, int64_t dv, int64_t window,
+                               int64_t maps) {
+  CHECK_CONTIG(out);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == q.scalar_type());
+  const int64_t T = q.size(0);
+  TORCH_CHECK(maps == 1 || maps == 2, "softmax_attention: one or two maps per head");
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == H * maps * dk, "q must be [T, H * maps * dk] rows");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv);
+  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dk <= 2048 && dv > 0 && dv <= 512 && window >= 0,
+              "softmax_attention: dk <= 2048, dv <= 512");
+  check_row_pages(q, kc, G * maps, dk, "softmax_attention (k)");
+  check_row_pages(q, vc, G, dv, "softmax_attention (v)");
+  TORCH_CHECK(kc.size(0) == vc.size(0));
+  SoftmaxArgs a;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == q.scalar_type() && gate->dim() == 2 && gate->size(0) == T &&
+                gate->size(1) == H && gate->stride(1) == 1, "gate must be [T, H] rows");
+    a.gp = gate->data_ptr();
+    a.gs = gate->stride(0);
+  }
+  return a;
+}
+
+void softmax_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc, Tensor block_tables,
+                       Tensor tok_seq, Tensor pos, int64_t H, int64_t G, int64_t dk, int64_t dv, double scale,
+                       int64_t window, int64_t maps, double lam, double unit_eps, double out_scale) {
+  const bool f32 = act_f32(q);
+  CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
+  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);
+  nga::launch_softmax_attention(out.data_ptr(), q.data_ptr(), q.stride(0), a.gp, a.gs, kc.data_ptr(), vc.data_ptr(),
+                                block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
+                                tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T, (int)H, (int)G, (int)dk,
+                                (int)dv, (float)scale, (int)window, (int)maps, (float)lam, (float)unit_eps,
+                                (float)out_scale, f32, cur_stream(q));
+}
+
+void hgrn2_scan(Tensor out, Tensor proj, Tensor f_bias, Tensor lower, Tensor state, int64_t H, int64_t d, int64_t dv,
+                c10::optional<Tensor> cu, Tensor slots, Tensor pos) {
+  const bool f32 = act_f32(proj);
+  CHECK_F32(out); CHECK_F32(f_bias); CHECK_F32(lower); CHECK_F32(state); CHECK_I32(slots); CHECK_I32(pos);
+  const int64_t T = proj.size(0);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(1) >= 2 * H * d + H * dv);
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv && pos.numel() == T);
+  TORCH_CHECK(f_bias.numel() == H * d && lower.numel() == H * d);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == d && state.size(3) == dv);
+  TORCH_CHECK(d <= nga::hgrn2_max_dim((int)dv), "hgrn2_scan: the per-head key size exceeds the kernel's register tile");
+  const int n = (int)slots.numel();
+  const int32_t* cp = nullptr;
+  if (cu.has_value()) {
+    CHECK_I32(*cu);
+    TORCH_CHECK(cu->numel() == n + 1);
+    cp = cu->data_ptr<int32_t>();
+  } else {
+    TORCH_CHECK(n == T, "hgrn2_scan: without cu every row is a segment");
+  }
+  TORCH_CHECK(nga::launch_hgrn2_scan(out.data_ptr<float>(), proj.data_ptr(), proj.stride(0), f_bias.data_ptr<float>(),
+                                     lower.data_ptr<float>(), state.data_ptr<float>(), (int)H, (int)d, (int)dv, cp,
+                                     slots.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), n, f32, cur_stream(proj)),
+              "hgrn2_scan: no kernel for these sizes");
+}
+
 }  // namespace
 
 
@@ -1186,6 +1344,15 @@ PYBIND11_MODULE(_C, m) {
   m.def("layernorm", checked("layernorm", &layernorm));
   m.def("add_layernorm", checked("add_layernorm", &add_layernorm));
   m.def("gelu_tanh_mul", checked("gelu_tanh_mul", &gelu_tanh_mul));
+  m.def("embed_rows", checked("embed_rows", &embed_rows));
+  m.def("rmsnorm_residual_next", checked("rmsnorm_residual_next", &rmsnorm_residual_next));
+  m.def("relu_sq", checked("relu_sq", &relu_sq));
+  m.def("softcap", checked("softcap", &softcap));
+  m.def("group_rmsnorm", checked("group_rmsnorm", &group_rmsnorm));
+  m.def("headnorm_cache", checked("headnorm_cache", &headnorm_cache));
+  m.def("softmax_attention", checked("softmax_attention", &softmax_attention));
+  m.def("hgrn2_scan", checked("hgrn2_scan", &hgrn2_scan));
+  m.def("softmax_attention_mfma_supported", [](int64_t dk, int64_t dv, int64_t group, int64_t maps) { return false; });
   m.def("embed_pos", checked("embed_pos", &embed_pos));
   m.def("rmsnorm_residual", checked("rmsnorm_residual", &rmsnorm_residual));
   m.def("rmsnorm_f32", checked("rmsnorm_f32", &rmsnorm_f32));

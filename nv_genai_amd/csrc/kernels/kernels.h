@@ -261,4 +261,30 @@ void launch_sigmoid_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
                                 int window, int keep_first, const float* r1, const float* r2, const float* pb,
                                 hipStream_t stream);
 
+// postnorm.hip: scaled embedding, sandwich norms with one gain or H, relu^2, soft cap, head norms
+void launch_embed_rows(float* x, const int32_t* ids, const void* embed, float scale, int64_t T, int H, int vocab,
+                       bool f32, hipStream_t stream);
+void launch_rmsnorm_residual_next(float* x, const void* y, int64_t y_stride, const float* w, int w_n, const float* nw,
+                                  int nw_n, float eps, int64_t T, int H, void* out, bool f32, hipStream_t stream);
+void launch_relu_sq(void* out, const void* in, int64_t n, bool f32, hipStream_t stream);
+void launch_softcap(float* z, int64_t n, float cap, hipStream_t stream);
+void launch_group_rmsnorm(void* out, const float* x, const float* w, int64_t T, int groups, int gs, float eps, bool f32,
+                          hipStream_t stream);
+
+// softmax_attention.hip: K [blocks, G * maps, 64, dk], V [blocks, G, 64, dv] pages, bf16 or fp32
+void launch_headnorm_cache(void* proj, int64_t stride, const int32_t* slots, void* kc, void* vc, int64_t T, int nq,
+                           int nk, int dk, int nv, int dv, float eps, const float* qw, const float* kw,
+                           const float* bias, const int32_t* pos, float coef, int every, bool f32, hipStream_t stream);
+void launch_softmax_attention(void* out, const void* q, int64_t q_stride, const void* gate, int64_t g_stride,
+                              const void* kc, const void* vc, const int32_t* block_tables, int max_blocks,
+                              const int32_t* tok_seq, const int32_t* pos, int64_t T, int H, int G, int dk, int dv,
+                              float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool f32,
+                              hipStream_t stream);
+
+// recurrent.hip
+int hgrn2_max_dim(int dv);
+bool launch_hgrn2_scan(float* out, const void* proj, int64_t stride, const float* f_bias, const float* lower,
+                       float* state, int H, int d, int dv, const int32_t* cu, const int32_t* slots, const int32_t* pos,
+                       int n_seg, bool f32, hipStream_t stream);
+
 }  // namespace nga

@@ -6,6 +6,13 @@
 //                     token earlier: a row of this step, a state slot, or zeros (position 0)
 //   shift_save        state[slot[i]] = x[last_row[i]] for every sequence of the step
 //   glu_gelu_tanh     [T, 2F] = [gate | up] -> gelu_tanh(gate) * up, any F, bf16 or fp32
+//   embed_rows        x[t]  = embed[id[t]] * scale                                (fp32 out)
+//   rmsnorm_residual_next   x[t] += rmsnorm(y[t]) * w, out[t] = rmsnorm(x[t]) * next_w: the
+//                     post-norm of one sub-layer and the pre-norm of the next in one pass
+//                     (weights of H elements or of one: a single gain)
+//   relu_sq           relu(x)^2
+//   softcap           z = cap * tanh(z / cap) on fp32 logits
+//   group_rmsnorm     RMS norm of each of G equal column groups of fp32 rows (heads)
 //
 // The residual, the norms and the shift interpolation are fp32 whatever the activation type T
 // (bf16 storage as uint16_t, or float). Memory-bound: one workgroup per row, columns strided
@@ -116,6 +123,88 @@ __global__ void __launch_bounds__(256) glu_gelu_tanh_kernel(T* __restrict__ out,
   }
 }
 
+template <typename T>
+__global__ void __launch_bounds__(256) embed_rows_kernel(float* __restrict__ x, const int32_t* __restrict__ ids,
+                                                         const T* __restrict__ embed, float scale, int H, int vocab) {
+  const int64_t row = blockIdx.x;
+  int id = ids[row];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // padding rows of a captured step
+  for (int c = threadIdx.x; c < H; c += blockDim.x) x[row * H + c] = ldf(embed + (int64_t)id * H + c) * scale;
+}
+
+// ws / nws: 1 when the weight has H elements, 0 when it is a single gain. Three passes over the
+// row: statistic of y, residual sum with the statistic of the new x, the next norm's output.
+template <typename T>
+__global__ void __launch_bounds__(256) rmsnorm_residual_next_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                                                    int64_t y_stride, const float* __restrict__ w,
+                                                                    int ws, const float* __restrict__ nw, int nws,
+                                                                    float eps, int H, T* __restrict__ out) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  float* xr = x + row * H;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float v = ldf(yr + c);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  float s2 = 0.f;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float v = xr[c] + ldf(yr + c) * r * w[c * ws];
+    xr[c] = v;
+    s2 += v * v;
+  }
+  s2 = block_sum(s2, red);
+  const float r2 = 1.0f / sqrtf(s2 / (float)H + eps);
+  // each thread re-reads only the columns it wrote itself
+  for (int c = threadIdx.x; c < H; c += blockDim.x) stf(out + row * H + c, xr[c] * r2 * nw[c * nws]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) relu_sq_kernel(T* __restrict__ out, const T* __restrict__ in, int64_t n) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const float v = fmaxf(ldf(in + i), 0.f);
+    stf(out + i, v * v);
+  }
+}
+
+__global__ void __launch_bounds__(256) relu_sq_bf16x8_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ in,
+                                                             int64_t n8) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n8; i += (int64_t)gridDim.x * blockDim.x) {
+    const u16x8 v = load8(in + i * 8);
+    u16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float f = fmaxf(bf2f(v[j]), 0.f);
+      o[j] = f2bf(f * f);
+    }
+    store8(out + i * 8, o);
+  }
+}
+
+__global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ z, int64_t n, float cap, float inv) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    z[i] = cap * tanhf(z[i] * inv);
+}
+
+// one wave per (row, group)
+template <typename T>
+__global__ void __launch_bounds__(256) group_rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                            const float* __restrict__ w, int64_t n_groups, int gs,
+                                                            float eps) {
+  const int64_t g = blockIdx.x * (int64_t)(blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (g >= n_groups) return;
+  const int lane = threadIdx.x & 63;
+  const float* xr = x + g * gs;
+  float ss = 0.f;
+  for (int c = lane; c < gs; c += 64) ss += xr[c] * xr[c];
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)gs + eps);
+  for (int c = lane; c < gs; c += 64) stf(out + g * gs + c, xr[c] * r * w[c]);
+}
+
 }  // namespace
 
 void launch_embed_pos(float* x, const int32_t* ids, const int32_t* pos, const void* embed, const void* ptab,
@@ -172,6 +261,61 @@ void launch_glu_gelu_tanh(void* out, const void* in, int64_t T, int F, bool f32,
     glu_gelu_tanh_kernel<float><<<dim3((unsigned)g), 256, 0, stream>>>((float*)out, (const float*)in, T, F);
   else
     glu_gelu_tanh_kernel<uint16_t><<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, T, F);
+}
+
+void launch_embed_rows(float* x, const int32_t* ids, const void* embed, float scale, int64_t T, int H, int vocab,
+                       bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    embed_rows_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(x, ids, (const float*)embed, scale, H, vocab);
+  else
+    embed_rows_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>(x, ids, (const uint16_t*)embed, scale, H, vocab);
+}
+
+void launch_rmsnorm_residual_next(float* x, const void* y, int64_t y_stride, const float* w, int w_n, const float* nw,
+                                  int nw_n, float eps, int64_t T, int H, void* out, bool f32, hipStream_t stream) {
+  if (T == 0) return;
+  const int ws = w_n == 1 ? 0 : 1, nws = nw_n == 1 ? 0 : 1;
+  if (f32)
+    rmsnorm_residual_next_kernel<float><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const float*)y, y_stride, w, ws, nw,
+                                                                              nws, eps, H, (float*)out);
+  else
+    rmsnorm_residual_next_kernel<uint16_t><<<dim3((unsigned)T), 256, 0, stream>>>(x, (const uint16_t*)y, y_stride, w,
+                                                                                 ws, nw, nws, eps, H, (uint16_t*)out);
+}
+
+void launch_relu_sq(void* out, const void* in, int64_t n, bool f32, hipStream_t stream) {
+  if (n == 0) return;
+  if (!f32 && n % 8 == 0) {
+    int64_t g = (n / 8 + 255) / 256;
+    if (g > 16384) g = 16384;
+    relu_sq_bf16x8_kernel<<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, n / 8);
+    return;
+  }
+  int64_t g = (n + 255) / 256;
+  if (g > 16384) g = 16384;
+  if (f32)
+    relu_sq_kernel<float><<<dim3((unsigned)g), 256, 0, stream>>>((float*)out, (const float*)in, n);
+  else
+    relu_sq_kernel<uint16_t><<<dim3((unsigned)g), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)in, n);
+}
+
+void launch_softcap(float* z, int64_t n, float cap, hipStream_t stream) {
+  if (n == 0) return;
+  int64_t g = (n + 255) / 256;
+  if (g > 16384) g = 16384;
+  softcap_kernel<<<dim3((unsigned)g), 256, 0, stream>>>(z, n, cap, 1.0f / cap);
+}
+
+void launch_group_rmsnorm(void* out, const float* x, const float* w, int64_t T, int groups, int gs, float eps, bool f32,
+                          hipStream_t stream) {
+  const int64_t ng = T * groups;
+  if (ng == 0) return;
+  const unsigned g = (unsigned)((ng + 3) / 4);
+  if (f32)
+    group_rmsnorm_kernel<float><<<dim3(g), 256, 0, stream>>>((float*)out, x, w, ng, gs, eps);
+  else
+    group_rmsnorm_kernel<uint16_t><<<dim3(g), 256, 0, stream>>>((uint16_t*)out, x, w, ng, gs, eps);
 }
 
 }  // namespace nga

@@ -10,7 +10,7 @@ real architecture on synthetic inputs.
 from __future__ import annotations
 
 from dataclasses import asdict, dataclass, field, replace
-from typing import Optional
+from typing import Optional, Sequence
 
 
 @dataclass(frozen=True)
@@ -369,3 +369,186 @@ def bidasun_uniform(layers: int, hidden: int, heads: int, kv_heads: int, dim: in
     blk = BlockSpec("attention", m, DenseMlpSpec(ff) if ff else None)
     return BidasunConfig(name=name, vocab_size=vocab_size, hidden=hidden, max_position=max_position, eps=eps,
                          blocks=(blk,) * layers)
+
+
+# ---------------------------------------------------------------------------------------------
+# Biruvik: a layer list whose entries choose between three mixers.
+@dataclass(frozen=True)
+class DiffAttentionSpec:
+    """Mixer ``attention`` of the Biruvik design: differential softmax attention. Every head has
+    two score maps (own q and k halves, shared v); ``o = a1 - lam * a2`` with one ``lam`` per
+    layer, unit RMS per head, times ``1 - diff``. Causal, GQA, per head-and-map RMS norm of q
+    and k, biases on q / k / v, no rotation; the query is scaled by
+    ``1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)`` at position p."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    diff: float
+    q_temp_coef: float
+    q_temp_every: int
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Mixer ``latent_attention``: keys and values are linear maps of one RMS-normed latent per
+    token (only the latent is cached), softmax over a sliding window (``window`` keys, the
+    query's own included; 0 = no limit), sigmoid output gate per head, no positions."""
+
+    heads: int
+    dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    window: int
+
+
+@dataclass(frozen=True)
+class Hgrn2Spec:
+    """Mixer ``hgrn2``: per head ``S <- diag(f) S + (1 - f) v^T``, ``o = S^T q`` with
+    ``q = silu(W_q h)`` and the forget gate ``f = l + (1 - l) sigmoid(W_f h + b)`` bounded from
+    below by ``l``; RMS norm of every head's output; fp32 state [heads, dim, vdim] per sequence."""
+
+    heads: int
+    dim: int
+    vdim: int
+
+
+@dataclass(frozen=True)
+class ReluSqMlpSpec:
+    ff: int
+    kind: str = "dense"     # down(relu(up x)^2)
+
+
+@dataclass(frozen=True)
+class BiruvikLayer:
+    type: str                 # "attention" | "latent_attention" | "hgrn2"
+    mixer: object
+    mlp: Optional[ReluSqMlpSpec] = None
+
+
+_BIRUVIK_MIXERS = ("attention", "latent_attention", "hgrn2")
+
+
+@dataclass(frozen=True)
+class BiruvikConfig:
+    """Biruvik: pre- and post-normed sub-layers on an fp32 residual stream
+    (``x += norm_b(sub(norm_a(x)))``, every norm an RMS norm with one gain), a scaled embedding,
+    no position table, a tanh soft cap on the logits. Every size and constant that can differ
+    between models comes from config.json (:meth:`from_dict`)."""
+
+    name: str = "biruvik"
+    vocab_size: int = 512
+    hidden: int = 128
+    eps: float = 1e-5
+    embed_scale: float = 1.0
+    logit_softcap: float = 0.0      # 0: none
+    blocks: tuple = ()
+    max_position: int = 1 << 20     # no position table: only the engine's bookkeeping is bounded
+    arch: str = "biruvik"
+    bos_id: int = 0
+    eos_ids: tuple = ()
+    chat_format: str = "plain"
+    is_moe: bool = False
+
+    @property
+    def layers(self) -> int:
+        return len(self.blocks)
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "biruvik") -> "BiruvikConfig":
+        blocks = []
+        for i, b in enumerate(d["layers"]):
+            t, m = b["type"], b["mixer"]
+            if t == "attention":
+                mixer = DiffAttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                          vdim=int(m["vdim"]), scale=float(m["scale"]), diff=float(m["diff"]),
+                                          q_temp_coef=float(m["q_temp"]["coef"]),
+                                          q_temp_every=int(m["q_temp"]["every"]))
+                if mixer.heads % mixer.kv_heads:
+                    raise ValueError(f"layer {i}: {mixer.heads} heads over {mixer.kv_heads} kv heads")
+                if mixer.q_temp_every < 1:
+                    raise ValueError(f"layer {i}: q_temp.every must be at least 1")
+            elif t == "latent_attention":
+                mixer = LatentAttentionSpec(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                            kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
+                                            window=int(m["mask"]["size"]))
+                if mixer.window < 1:
+                    raise ValueError(f"layer {i}: a window holds at least the query's own position")
+            elif t == "hgrn2":
+                mixer = Hgrn2Spec(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {t!r} (known: {_BIRUVIK_MIXERS})")
+            mlp = b.get("mlp")
+            if mlp is not None:
+                if mlp.get("kind", "dense") != "dense":
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {mlp['kind']!r}")
+                mlp = ReluSqMlpSpec(ff=int(mlp["ff"]))
+            blocks.append(BiruvikLayer(type=t, mixer=mixer, mlp=mlp))
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), eps=float(d["norm"]["eps"]),
+                   embed_scale=float(d["embedding"]["scale"]), logit_softcap=float(d.get("logit_softcap") or 0.0),
+                   blocks=tuple(blocks))
+
+    def to_json_dict(self) -> dict:
+        """The config.json form (inverse of :meth:`from_dict`)."""
+        layers = []
+        for b in self.blocks:
+            m = b.mixer
+            if b.type == "attention":
+                mx = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "scale": m.scale,
+                      "diff": m.diff, "q_temp": {"coef": m.q_temp_coef, "every": m.q_temp_every}}
+            elif b.type == "latent_attention":
+                mx = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim, "kv_rank": m.kv_rank, "scale": m.scale,
+                      "mask": {"size": m.window}}
+            else:
+                mx = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim}
+            layers.append({"type": b.type, "mixer": mx,
+                           "mlp": None if b.mlp is None else {"kind": b.mlp.kind, "ff": b.mlp.ff}})
+        return {"architecture": "Biruvik", "vocab": self.vocab_size, "width": self.hidden,
+                "embedding": {"scale": self.embed_scale}, "norm": {"eps": self.eps},
+                "logit_softcap": self.logit_softcap, "layers": layers}
+
+    def num_params(self) -> int:
+        H = self.hidden
+        n = 2 * self.vocab_size * H + 1
+        for b in self.blocks:
+            m = b.mixer
+            n += 2
+            if b.type == "attention":
+                n += (H + 1) * (2 * m.heads * m.dim + 2 * m.kv_heads * m.dim + m.kv_heads * m.vdim) + 6 * m.dim
+                n += H * m.heads * m.vdim
+            elif b.type == "latent_attention":
+                n += H * (m.heads * m.dim + m.kv_rank + m.heads) + m.kv_rank
+                n += m.kv_rank * m.heads * (m.dim + m.vdim) + H * m.heads * m.vdim
+            else:
+                n += H * (2 * m.heads * m.dim + m.heads * m.vdim) + 2 * m.heads * m.dim + m.vdim
+                n += H * m.heads * m.vdim
+            if b.mlp is not None:
+                n += 2 * H * b.mlp.ff + 2
+        return n
+
+    def to_dict(self):
+        return asdict(self)
+
+
+def biruvik_layers(pattern: Sequence[str], hidden: int, heads: int, kv_heads: int, dim: int, vdim: int, ff: int,
+                   window: int = 1024, kv_rank: int = 512, diff: float = 0.25, q_temp=(0.1, 1024),
+                   vocab_size: int = 32768, embed_scale: float = 1.0, logit_softcap: float = 30.0,
+                   eps: float = 1e-5, name: str = "biruvik") -> BiruvikConfig:
+    """A Biruvik config from a pattern of mixer types with the same sizes in every layer
+    (benchmarks, tests)."""
+    blocks = []
+    for t in pattern:
+        if t == "attention":
+            m = DiffAttentionSpec(heads, kv_heads, dim, vdim, dim ** -0.5, diff, float(q_temp[0]), int(q_temp[1]))
+        elif t == "latent_attention":
+            m = LatentAttentionSpec(heads, dim, vdim, kv_rank, dim ** -0.5, window)
+        elif t == "hgrn2":
+            m = Hgrn2Spec(heads, dim, vdim)
+        else:
+            raise ValueError(f"unknown mixer type {t!r}")
+        blocks.append(BiruvikLayer(t, m, ReluSqMlpSpec(ff) if ff else None))
+    return BiruvikConfig(name=name, vocab_size=vocab_size, hidden=hidden, eps=eps, embed_scale=embed_scale,
+                         logit_softcap=logit_softcap, blocks=tuple(blocks))

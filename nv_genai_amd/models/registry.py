@@ -14,7 +14,7 @@ from typing import Callable, Dict, Optional, Tuple
 
 import torch
 
-from .config import LLAMA_PRESETS, BidasunConfig, LlamaConfig
+from .config import LLAMA_PRESETS, BidasunConfig, BiruvikConfig, LlamaConfig
 
 # design name (lower case) -> (config builder from the config.json dict, model class loader)
 _REGISTRY: Dict[str, Tuple[Callable[[dict], object], Callable[[], type]]] = {}
@@ -28,6 +28,12 @@ def _bidasun_class():
     from .bidasun import BidasunModel
 
     return BidasunModel
+
+
+def _biruvik_class():
+    from .biruvik import BiruvikModel
+
+    return BiruvikModel
 
 
 def _llama_class():
@@ -66,6 +72,7 @@ def _hf_decoder_config(d: dict) -> LlamaConfig:
 
 
 register("bidasun", BidasunConfig.from_dict, _bidasun_class)
+register("biruvik", BiruvikConfig.from_dict, _biruvik_class)
 for _t in _HF_ARCH:
     register(_t, _hf_decoder_config, _llama_class)
 
@@ -74,6 +81,8 @@ def model_class_for(cfg) -> type:
     """Model class of a config object."""
     if isinstance(cfg, BidasunConfig):
         return _bidasun_class()
+    if isinstance(cfg, BiruvikConfig):
+        return _biruvik_class()
     if isinstance(cfg, LlamaConfig):
         return _llama_class()
     raise ValueError(f"no model class for {type(cfg).__name__}")

@@ -462,6 +462,169 @@ def sigmoid_attention_rows(q, gate, kc, vc, block_tables, tok_seq, pos, Hq: int,
     return out
 
 
+# ------------------------------------------------------------------------- scaled embedding, sandwich norms, relu^2, soft cap
+def embed_rows(ids: torch.Tensor, embed: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """fp32 residual rows ``embed[id] * scale`` (table bf16 or fp32)."""
+    if not _gpu(embed):
+        return ref.embed_rows(ids, embed, scale)
+    x = torch.empty(ids.numel(), embed.shape[1], dtype=torch.float32, device=embed.device)
+    kernels().embed_rows(x, ids, embed, float(scale))
+    return x
+
+
+def rmsnorm_residual_next_(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float, next_w: torch.Tensor,
+                           dtype: torch.dtype) -> torch.Tensor:
+    """Sandwich-norm step on an fp32 stream: ``x += rmsnorm(y) * w`` in place, and returns
+    ``rmsnorm(x) * next_w`` (the next sub-layer's input) in ``dtype`` from the same launch. The
+    weights are fp32 with H elements or one (a single gain for all coordinates)."""
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    if not _gpu(x):
+        ref.rmsnorm_residual_next_(x, y, w, eps, next_w, out)
+        return out
+    kernels().rmsnorm_residual_next(x, y, w, float(eps), next_w, out)
+    return out
+
+
+def relu_sq(x: torch.Tensor) -> torch.Tensor:
+    """relu(x)^2, bf16 or fp32."""
+    if not _gpu(x):
+        return ref.relu_sq(x)
+    out = torch.empty_like(x)
+    kernels().relu_sq(out, x)
+    return out
+
+
+def softcap_(z: torch.Tensor, cap: float) -> torch.Tensor:
+    """fp32 logits in place: ``cap * tanh(z / cap)``."""
+    if not _gpu(z):
+        return ref.softcap_(z, cap)
+    kernels().softcap(z, float(cap))
+    return z
+
+
+def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float, dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of each of ``groups`` equal column groups of fp32 rows (one weight per element of
+    a group, shared by the groups), written in ``dtype``."""
+    if not _gpu(x):
+        return ref.group_rmsnorm(x, w, groups, eps, dtype)
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    kernels().group_rmsnorm(out, x, w, int(groups), float(eps))
+    return out
+
+
+# ------------------------------------------------------------------------- softmax attention with head maps (row-major pages)
+def headnorm_cache_(proj, slots, kc, vc, nq: int, nk: int, dk: int, nv: int, dv: int, eps: float, q_w=None,
+                    k_w=None, bias=None, pos=None, temp_coef: float = 0.0, temp_every: int = 1):
+    """Projection rows ``[q: nq heads of dk | k: nk heads of dk | v: nv heads of dv | ...]`` in
+    place: add ``bias`` (fp32, over the q | k | v columns), RMS-normalise every q head with
+    ``q_w`` [dk] and every k head with ``k_w`` [dk] (None: that part is left as it is), scale q
+    by ``1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)``, and write k / v into the
+    token's page slot: K [blocks, nk, 64, dk], V [blocks, nv, 64, dv] (``slots`` < 0: no write;
+    ``vc`` None with nv = 0)."""
+    if not _gpu(proj):
+        return ref.headnorm_cache_(proj, slots, kc, vc, nq, nk, dk, nv, dv, eps, q_w, k_w, bias, pos, temp_coef,
+                                   temp_every)
+    kernels().headnorm_cache(proj, slots, kc, vc, nq, nk, dk, nv, dv, float(eps), q_w, k_w, bias, pos,
+                             float(temp_coef), int(temp_every))
+    return proj
+
+
+def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk: int, dv: int, scale: float,
+                      window: int = 0, maps: int = 1, lam: float = 0.0, unit_eps: Optional[float] = None,
+                      out_scale: float = 1.0, gate=None, out=None):
+    """Softmax attention of token rows (prompt portions and single-token rows alike) over row-
+    major pages K [blocks, G * maps, 64, dk], V [blocks, G, 64, dv]. The query at position i
+    sees keys ``j <= i`` (``window`` > 0: and ``i - j < window``). ``maps`` (1 or 2) score maps per
+    head: q head (h, m) is column block ``h * maps + m``, its keys are k head
+    ``(h // (H / G)) * maps + m``, both maps read v head ``h // (H / G)``; two maps combine as
+    ``a_0 - lam * a_1`` (differential attention). ``unit_eps``: divide every head's output by its
+    root mean square (eps inside the root) and multiply by ``out_scale``. ``gate`` [T, H]: the
+    head outputs are multiplied by ``sigmoid(gate)``. ``tok_seq[t]`` is the block-table row of
+    token t, ``pos[t]`` its position (negative: padding row, zeros out). Scores, softmax and
+    accumulation are fp32."""
+    if not _gpu(q):
+        return ref.softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam,
+                                     unit_eps, out_scale, gate)
+    if out is None:
+        out = torch.empty(q.shape[0], H * dv, dtype=q.dtype, device=q.device)
+    kernels().softmax_attention(out, q, gate, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, float(scale),
+                                int(window), int(maps), float(lam), -1.0 if unit_eps is None else float(unit_eps),
+                                float(out_scale))
+    return out
+
+
+def softmax_attention_mfma_ok(q: torch.Tensor, dk: int, dv: int, group: int = 1, maps: int = 1) -> bool:
+    """The MFMA softmax attention kernels take bf16 GPU rows with dk, dv multiples of 32 up to
+    the sizes the kernels were instantiated for."""
+    return (_gpu(q) and q.dtype == torch.bfloat16 and have_kernels()
+            and bool(kernels().softmax_attention_mfma_supported(int(dk), int(dv), int(group), int(maps))))
+
+
+def _rows_of_portions(cu_q, ctx_lens, T: int, dev):
+    """(block-table row, position) of every token row of portions laid out by ``cu_q``."""
+    n = (cu_q[1:] - cu_q[:-1]).long()
+    seq = torch.repeat_interleave(torch.arange(n.numel(), device=dev), n, output_size=T)
+    pos = (ctx_lens.long() - n - cu_q[:-1].long())[seq] + torch.arange(T, device=dev)
+    return seq.int(), pos.int()
+
+
+def softmax_attention_prefill(q, kc, vc, block_tables, cu_q, ctx_lens, max_q_len: int, H: int, G: int, dk: int,
+                              dv: int, scale: float, window: int = 0, maps: int = 1, lam: float = 0.0,
+                              unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None):
+    """:func:`softmax_attention` of prompt portions on MFMA tiles: sequence b owns token rows
+    ``[cu_q[b], cu_q[b + 1])``, the last ones of its ``ctx_lens[b]`` keys. Rows the tile kernel
+    does not take (fp32, other head sizes, CPU) run the row form."""
+    if not softmax_attention_mfma_ok(q, dk, dv, H // G, maps):
+        seq, pos = _rows_of_portions(cu_q, ctx_lens, q.shape[0], q.device)
+        return softmax_attention(q, kc, vc, block_tables, seq, pos, H, G, dk, dv, scale, window, maps, lam, unit_eps,
+                                 out_scale, gate, out=out)
+    if out is None:
+        out = torch.empty(q.shape[0], H * dv, dtype=q.dtype, device=q.device)
+    kernels().softmax_attention_prefill(out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, int(max_q_len), H, G, dk,
+                                        dv, float(scale), int(window), int(maps), float(lam),
+                                        -1.0 if unit_eps is None else float(unit_eps), float(out_scale))
+    return out
+
+
+def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk: int, dv: int, scale: float,
+                           max_ctx: int, window: int = 0, maps: int = 1, lam: float = 0.0,
+                           unit_eps: Optional[float] = None, out_scale: float = 1.0, gate=None, out=None):
+    """:func:`softmax_attention` of single-token rows (decode rows; any rows work) on the page-
+    parallel MFMA kernel: the query heads that share a KV head are the columns of one tile, so a
+    page is read once per group; the visible pages of a row are split over several workgroups
+    whose (max, sum, accumulator) partials a second kernel merges, which also combines the maps,
+    normalises and gates. ``max_ctx`` bounds the rows' positions (launch shape)."""
+    if not softmax_attention_mfma_ok(q, dk, dv, H // G, maps):
+        return softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window, maps, lam,
+                                 unit_eps, out_scale, gate, out=out)
+    C = kernels()
+    T = q.shape[0]
+    parts = int(C.softmax_decode_parts(max(T, 1), G * maps, int(max_ctx), int(window)))
+    ws = torch.empty(T * H * maps * parts * (dv + 2), dtype=torch.float32, device=q.device)
+    if out is None:
+        out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    C.softmax_attention_decode(out, ws, parts, q, gate, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv,
+                               float(scale), int(window), int(maps), float(lam),
+                               -1.0 if unit_eps is None else float(unit_eps), float(out_scale))
+    return out
+
+
+# ------------------------------------------------------------------------- gated linear recurrence
+def hgrn2_scan(proj, f_bias, lower, state, H: int, d: int, dv: int, cu, slots, pos) -> torch.Tensor:
+    """HGRN2 recurrence over a step's rows. ``proj`` rows ``[q (H*d) | f (H*d) | v (H*dv)]`` hold
+    pre-activations: ``q = silu(q)``, ``f = lower + (1 - lower) * sigmoid(f + f_bias)`` (fp32).
+    Segment b is rows ``cu[b] .. cu[b + 1]`` (``cu`` None: row b alone) of one sequence; its state
+    [H, d, dv] (fp32) comes from ``state[slots[b]]``, or zeros when the segment starts at
+    position 0 (``pos`` per row) — a reused slot needs no clearing — and goes back there after
+    ``S <- diag(f) S + (1 - f) v^T``, ``o = S^T q`` per row. ``slots[b]`` < 0: nothing is read or
+    kept. Returns the un-normalised fp32 outputs [T, H*dv]."""
+    if not _gpu(proj):
+        return ref.hgrn2_scan(proj, f_bias, lower, state, H, d, dv, cu, slots, pos)
+    out = torch.empty(proj.shape[0], H * dv, dtype=torch.float32, device=proj.device)
+    kernels().hgrn2_scan(out, proj, f_bias, lower, state, H, d, dv, cu, slots, pos)
+    return out
+
+
 class DecodeWorkspace:
     """Split-K partition buffers for decode attention, sized for (max_seqs, Hq, max_ctx).
 

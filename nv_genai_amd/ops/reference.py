@@ -513,3 +513,135 @@ def sigmoid_attention(q, gate, kc, vc, block_tables, tok_seq, pos, Hq, Hkv, dk, 
     if gate is not None:
         out = out * torch.sigmoid(gate.float())
     return out.to(q.dtype)
+
+
+# ------------------------------------------------------------------------- softmax attention with head maps,
+# gated linear recurrence, per-head norms (row-major pages: K [blocks, heads, 64, dk], V [blocks, heads, 64, dv])
+def embed_rows(ids, embed, scale=1.0):
+    """fp32 rows embed[id] * scale."""
+    return embed[ids.long()].float() * scale
+
+
+def rmsnorm_residual_next_(x, y, w, eps, next_w, out):
+    """x (fp32, in place) += rmsnorm(y) * w, then out = rmsnorm(x) * next_w (weights of one or H
+    elements)."""
+    yf = y.float()
+    x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * w)
+    out.copy_(x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * next_w)
+    return x
+
+
+def relu_sq(x):
+    r = torch.relu(x.float())
+    return (r * r).to(x.dtype)
+
+
+def softcap_(z, cap):
+    return z.copy_(cap * torch.tanh(z / cap))
+
+
+def query_temperature(pos, coef, every):
+    """1 + coef * ln(floor((p + 1) / every) + 1) per position (fp32)."""
+    return 1.0 + coef * torch.log((torch.div(pos.long() + 1, every, rounding_mode="floor") + 1).float())
+
+
+def headnorm_cache_(proj, slots, kc, vc, nq, nk, dk, nv, dv, eps, q_w=None, k_w=None, bias=None, pos=None,
+                    temp_coef=0.0, temp_every=1):
+    """Rows [q: nq heads of dk | k: nk heads of dk | v: nv heads of dv | ...]: add ``bias``, RMS-
+    normalise every q head (``q_w``) and every k head (``k_w``) over its dk elements, scale q by
+    the query temperature of its position, write q and k back in place, and k / v into the
+    token's page slot."""
+    n0, n1, n2 = nq * dk, (nq + nk) * dk, (nq + nk) * dk + nv * dv
+    T = proj.shape[0]
+    seg = proj[:, :n2].float()
+    if bias is not None:
+        seg = seg + bias
+    q, k, v = seg[:, :n0].reshape(T, nq, dk), seg[:, n0:n1].reshape(T, nk, dk), seg[:, n1:n2]
+    if q_w is not None and nq:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_w
+    if temp_coef != 0.0 and nq:
+        q = q * query_temperature(pos, temp_coef, temp_every)[:, None, None]
+    if k_w is not None and nk:
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_w
+    proj[:, :n0] = q.reshape(T, n0).to(proj.dtype)
+    proj[:, n0:n1] = k.reshape(T, n1 - n0).to(proj.dtype)
+    proj[:, n1:n2] = v.to(proj.dtype)
+    sl = slots.long()
+    ok = sl >= 0
+    BS = kc.shape[2]
+    blk, off = sl[ok] // BS, sl[ok] % BS
+    if nk:
+        kc[blk, :, off, :] = k[ok].to(kc.dtype)
+    if nv:
+        vc[blk, :, off, :] = v[ok].reshape(-1, nv, dv).to(vc.dtype)
+    return proj
+
+
+def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv, scale, window=0, maps=1, lam=0.0,
+                      unit_eps=None, out_scale=1.0, gate=None):
+    """Softmax attention of token rows over row-major pages, one row at a time. ``maps`` score
+    maps per head (q head (h, m) at column (h * maps + m) * dk, k head (h // (H / G)) * maps + m,
+    v head h // (H / G)), combined as a_0 - lam * a_1; optional unit RMS per head (times
+    ``out_scale``) and a per-head sigmoid gate."""
+    T = q.shape[0]
+    out = torch.zeros(T, H, dv, dtype=torch.float32, device=q.device)
+    BS = kc.shape[2]
+    rep = H // G
+    vh = torch.arange(H, device=q.device) // rep
+    qf = q.float().view(T, H, maps, dk)
+    for t in range(T):
+        i = int(pos[t])
+        if i < 0:
+            continue
+        bt = block_tables[int(tok_seq[t])]
+        lo = max(0, i - window + 1) if window else 0
+        j = torch.arange(lo, i + 1, device=q.device)
+        blk, off = bt[j // BS].long(), j % BS
+        k = kc[blk, :, off, :].float().view(-1, G, maps, dk)[:, vh]     # [n, H, maps, dk]
+        v = vc[blk, :, off, :].float()[:, vh]                          # [n, H, dv]
+        s = torch.einsum("hmd,nhmd->hmn", qf[t], k) * scale
+        a = torch.einsum("hmn,nhd->hmd", torch.softmax(s, -1), v)
+        out[t] = a[:, 0] - lam * a[:, 1] if maps == 2 else a[:, 0]
+    if unit_eps is not None:
+        out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + unit_eps) * out_scale
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[:, :, None]
+    return out.reshape(T, H * dv).to(q.dtype)
+
+
+def hgrn2_scan(proj, f_bias, lower, state, H, d, dv, cu, slots, pos):
+    """Rows [q (H*d) | f (H*d) | v (H*dv)] of pre-activations -> fp32 [T, H*dv]:
+    q = silu(q), f = lower + (1 - lower) * sigmoid(f + f_bias); per segment (rows cu[b] ..
+    cu[b + 1], or one row each when ``cu`` is None) S <- f S + (1 - f) v^T from the state slot
+    (zeros when the segment starts at position 0), o = S^T q; the slot takes the last S."""
+    T = proj.shape[0]
+    n = slots.numel()
+    qd = H * d
+    pf = proj.float()
+    q = torch.nn.functional.silu(pf[:, :qd]).view(T, H, d)
+    f = (lower + (1.0 - lower) * torch.sigmoid(pf[:, qd:2 * qd] + f_bias)).view(T, H, d)
+    v = pf[:, 2 * qd:2 * qd + H * dv].reshape(T, H, dv)
+    out = torch.zeros(T, H, dv, dtype=torch.float32, device=proj.device)
+    for b in range(n):
+        t0, t1 = (b, b + 1) if cu is None else (int(cu[b]), int(cu[b + 1]))
+        if t1 <= t0:
+            continue
+        sl = int(slots[b])
+        if int(pos[t0]) == 0 or sl < 0:
+            S = torch.zeros(H, d, dv, dtype=torch.float32, device=proj.device)
+        else:
+            S = state[sl].clone()
+        for t in range(t0, t1):
+            S = f[t][:, :, None] * S + (1.0 - f[t])[:, :, None] * v[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        if sl >= 0:
+            state[sl] = S
+    return out.reshape(T, H * dv)
+
+
+def group_rmsnorm(x, w, groups, eps, dtype):
+    """RMS norm of every one of ``groups`` equal column groups of fp32 rows, weight per element
+    of a group, written in ``dtype``."""
+    T = x.shape[0]
+    xg = x.view(T, groups, -1)
+    return (xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps) * w).reshape(T, -1).to(dtype)

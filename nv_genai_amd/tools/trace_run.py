@@ -61,7 +61,8 @@ def main(argv=None) -> int:
     torch.backends.cuda.matmul.allow_tf32 = False
     mcfg, _ = read_config(a.model)
     pages = max(1, a.max_tokens // 64)
-    max_len = int(getattr(mcfg, "max_position", 8192))
+    # no request outgrows the pool, whatever the model's own limit
+    max_len = min(int(getattr(mcfg, "max_position", 8192)), max(64, -(-a.max_tokens // 64) * 64))
     sizes = tuple(b for b in (1, 2, 4, 8, 16, 32) if b <= a.slots)
     eng = LLMEngine(EngineConfig(model=a.model, dtype=a.dtype, max_num_seqs=a.slots,
                                  max_batched_tokens=max(a.max_tokens, 64), max_model_len=max_len,
