@@ -1266,6 +1266,47 @@ void softmax_attention(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor 
                                 (float)out_scale, f32, cur_stream(q));
 }
 
+// prompt portions on the MFMA kernel (bf16): sequence b owns rows [cu_q[b], cu_q[b + 1]) of q / gate / out,
+// the last ones of its ctx_lens[b] keys
+void softmax_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate, Tensor kc, Tensor vc,
+                               Tensor block_tables, Tensor cu_q, Tensor ctx_lens, int64_t max_q_len, int64_t H,
+                               int64_t G, int64_t dk, int64_t dv, double scale, int64_t window, int64_t maps, double lam,
+                               double unit_eps, double out_scale) {
+  CHECK_BF16(q); CHECK_BF16(out); CHECK_I32(block_tables); CHECK_I32(cu_q); CHECK_I32(ctx_lens);
+  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps);
+  TORCH_CHECK(nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)(H / G), (int)maps),
+              "softmax_attention_prefill: head sizes the MFMA kernel does not take");
+  TORCH_CHECK(q.stride(0) % 8 == 0 && (uintptr_t)q.data_ptr() % 16 == 0, "q rows must be 16-B aligned");
+  const int64_t B = ctx_lens.numel();
+  TORCH_CHECK(cu_q.numel() == B + 1 && block_tables.dim() == 2 && block_tables.size(0) >= B && max_q_len >= 0);
+  nga::launch_softmax_attention_mfma(bfp(out), bfp(q), q.stride(0), (const uint16_t*)a.gp, a.gs, bfp(kc), bfp(vc),
+                                     block_tables.data_ptr<int32_t>(), (int)block_tables.size(1),
+                                     cu_q.data_ptr<int32_t>(), ctx_lens.data_ptr<int32_t>(), (int)B, (int)max_q_len,
+                                     (int)H, (int)G, (int)dk, (int)dv, (float)scale, (int)window, (int)maps, (float)lam,
+                                     (float)unit_eps, (float)out_scale, cur_stream(q));
+}
+
+// single-token rows on the MFMA kernel (bf16): ws is the fp32 partial workspace [T, H, maps, 4 * parts, dv + 4]
+void softmax_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c10::optional<Tensor> gate, Tensor kc,
+                              Tensor vc, Tensor block_tables, Tensor tok_seq, Tensor pos, int64_t H, int64_t G,
+                              int64_t dk, int64_t dv, double scale, int64_t window, int64_t maps, double lam,
+                              double unit_eps, double out_scale) {
+  CHECK_BF16(q); CHECK_BF16(out); CHECK_F32(ws); CHECK_I32(block_tables); CHECK_I32(tok_seq); CHECK_I32(pos);
+  const SoftmaxArgs a = check_softmax_args(out, q, gate, kc, vc, H, G, dk, dv, window, maps);
+  TORCH_CHECK(nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)(H / G), (int)maps),
+              "softmax_attention_decode: head sizes the MFMA kernel does not take");
+  TORCH_CHECK(q.stride(0) % 8 == 0 && (uintptr_t)q.data_ptr() % 16 == 0, "q rows must be 16-B aligned");
+  const int64_t T = q.size(0);
+  TORCH_CHECK(parts >= 1 && parts <= 64 && ws.numel() >= T * H * maps * 4 * parts * (dv + 4) &&
+              (uintptr_t)ws.data_ptr() % 16 == 0);
+  TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);
+  nga::launch_softmax_decode_mfma(bfp(out), ws.data_ptr<float>(), (int)parts, bfp(q), q.stride(0),
+                                  (const uint16_t*)a.gp, a.gs, bfp(kc), bfp(vc), block_tables.data_ptr<int32_t>(),
+                                  (int)block_tables.size(1), tok_seq.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), T,
+                                  (int)H, (int)G, (int)dk, (int)dv, (float)scale, (int)window, (int)maps, (float)lam,
+                                  (float)unit_eps, (float)out_scale, cur_stream(q));
+}
+
 void hgrn2_scan(Tensor out, Tensor proj, Tensor f_bias, Tensor lower, Tensor state, int64_t H, int64_t d, int64_t dv,
                 c10::optional<Tensor> cu, Tensor slots, Tensor pos) {
   const bool f32 = act_f32(proj);
@@ -1352,7 +1393,14 @@ PYBIND11_MODULE(_C, m) {
   m.def("headnorm_cache", checked("headnorm_cache", &headnorm_cache));
   m.def("softmax_attention", checked("softmax_attention", &softmax_attention));
   m.def("hgrn2_scan", checked("hgrn2_scan", &hgrn2_scan));
-  m.def("softmax_attention_mfma_supported", [](int64_t dk, int64_t dv, int64_t group, int64_t maps) { return false; });
+  m.def("softmax_attention_mfma_supported", [](int64_t dk, int64_t dv, int64_t group, int64_t maps) {
+    return nga::softmax_attention_mfma_supported((int)dk, (int)dv, (int)group, (int)maps);
+  });
+  m.def("softmax_attention_prefill", checked("softmax_attention_prefill", &softmax_attention_prefill));
+  m.def("softmax_attention_decode", checked("softmax_attention_decode", &softmax_attention_decode));
+  m.def("softmax_decode_parts", [](int64_t rows, int64_t G, int64_t max_ctx, int64_t window) {
+    return (int64_t)nga::softmax_decode_parts((int)rows, (int)G, (int)max_ctx, (int)window);
+  });
   m.def("embed_pos", checked("embed_pos", &embed_pos));
   m.def("rmsnorm_residual", checked("rmsnorm_residual", &rmsnorm_residual));
   m.def("rmsnorm_f32", checked("rmsnorm_f32", &rmsnorm_f32));

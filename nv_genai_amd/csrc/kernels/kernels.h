@@ -281,6 +281,20 @@ void launch_softmax_attention(void* out, const void* q, int64_t q_stride, const 
                               float scale, int window, int maps, float lam, float unit_eps, float out_scale, bool f32,
                               hipStream_t stream);
 
+bool softmax_attention_mfma_supported(int dk, int dv, int group, int maps);
+void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_stride, const uint16_t* gate,
+                                   int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
+                                   const int32_t* block_tables, int max_blocks, const int32_t* cu_q,
+                                   const int32_t* ctx_lens, int B, int max_q_len, int H, int G, int dk, int dv,
+                                   float scale, int window, int maps, float lam, float unit_eps, float out_scale,
+                                   hipStream_t stream);
+int softmax_decode_parts(int rows, int G, int max_ctx, int window);
+void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
+                                const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
+                                const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
+                                const int32_t* pos, int64_t T, int H, int G, int dk, int dv, float scale, int window,
+                                int maps, float lam, float unit_eps, float out_scale, hipStream_t stream);
+
 // recurrent.hip
 int hgrn2_max_dim(int dv);
 bool launch_hgrn2_scan(float* out, const void* proj, int64_t stride, const float* f_bias, const float* lower,

@@ -196,7 +196,574 @@ __global__ void __launch_bounds__(64) softmax_attention_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// MFMA form for prompt portions (bf16). Workgroup = 4 waves = 64 query rows of one sequence and
+// one head; each wave owns 16 rows (the 16 columns of its mfma_f32_16x16x32_bf16 tiles) and runs
+// all maps of the head, so a V page is staged once for both maps. Per 64-key page the workgroup
+// stages K [maps][64][DK] in LDS (16-B chunks XOR-swizzled by row) and V transposed, V^T [DV][64]:
+// a thread loads 4 keys x 8 value columns with 16-B loads, transposes them in registers and
+// writes 8 rows x 4 keys with 8-byte stores. Every wave computes S^T = K . Q^T with the key rows
+// permuted so that lane (query, h) ends up holding keys 32g + 8h .. + 7 of the page in its
+// accumulators - exactly the B operand of O^T += V^T . P^T, so the weights never move between
+// lanes. The softmax runs per query column in the exp2 domain: the running maximum and sum are
+// reduced over the lane's 16 scores and the 4 lanes of its column; accumulators are rescaled
+// when the maximum moves. Pages visited: those the block's windows cover.
+__device__ __forceinline__ int sm_row_swz(int row) { return (row & 3) | (((row >> 3) & 3) << 2); }
+
+struct SmMfmaParams {
+  uint16_t* out;             // [T, H * DV]
+  const uint16_t* q;         // row stride q_stride, head (h, m) at (h * MAPS + m) * DK
+  const uint16_t* gate;      // row stride g_stride, one value per head (nullptr: none)
+  const uint16_t* kc;
+  const uint16_t* vc;
+  const int32_t* block_tables;
+  const int32_t* cu_q;       // [B + 1] token rows of each sequence in this launch
+  const int32_t* ctx_lens;   // [B] keys of each sequence after this step (its rows are the last ones)
+  int64_t q_stride, g_stride;
+  int max_blocks, H, G, window;
+  float scale_log2, lam, unit_eps, out_scale;
+};
+
+template <int DK, int DV, int MAPS>
+__global__ void __launch_bounds__(256) softmax_attention_mfma_kernel(const SmMfmaParams P) {
+  constexpr int KT = 64;
+  constexpr int NCH_K = DK / 8;
+  constexpr int DS = DK / 32;
+  constexpr int DT = DV / 16;
+  constexpr int PER_K = DK / 32;           // 16-B chunks per thread per K page
+  constexpr int VBLK = (2 * DV + 255) / 256;   // (4 keys x 8 columns) blocks per thread per V page
+  constexpr int SWS = NCH_K >= 16 ? 0 : NCH_K == 8 ? 1 : 2;
+  extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
+  uint16_t* k_s = sm_lds;                       // [MAPS][KT * DK]
+  uint16_t* v_s = sm_lds + MAPS * KT * DK;      // [DV * KT]
+  const int tile = blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
+  const int q0 = P.cu_q[b], qlen = P.cu_q[b + 1] - q0;
+  if (tile * 64 >= qlen) return;
+  const int ctx = P.ctx_lens[b];
+  const int g = hq / (P.H / P.G);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, h = lane >> 4;
+  const int W = P.window;
+
+  int r = tile * 64 + w * 16 + col;
+  const bool row_ok = r < qlen;
+  if (!row_ok) r = qlen - 1;
+  const int qpos = ctx - qlen + r;
+  bf16x8 qf[MAPS][DS];
+  {
+    const uint16_t* qp = P.q + (int64_t)(q0 + r) * P.q_stride + (int64_t)hq * MAPS * DK;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+      for (int s2 = 0; s2 < DS; ++s2) qf[m][s2] = as_bf16x8(load8(qp + m * DK + 32 * s2 + 8 * h));
+  }
+  const int qpos_lo = ctx - qlen + tile * 64;
+  const int qpos_hi = ctx - qlen + min(qlen - 1, tile * 64 + 63);
+  const int lo_min = W > 0 ? max(0, qpos_lo - W + 1) : 0;
+  const int t_first = lo_min / KT, t_last = qpos_hi / KT;
+  const float fW = W > 0 ? (float)W : 3.0e38f;
+  // positions of this wave's first and last rows
+  const int wq_lo = ctx - qlen + min(qlen - 1, tile * 64 + w * 16);
+  const int wq_hi = ctx - qlen + min(qlen - 1, tile * 64 + w * 16 + 15);
+
+  f32x4 o[MAPS][DT];
+  float mrun[MAPS], lrun[MAPS];
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) {
+    mrun[m] = -INFINITY;
+    lrun[m] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[m][dt] = (f32x4)(0.f);
+  }
+
+  for (int t = t_first; t <= t_last; ++t) {
+    const int64_t blk = P.block_tables[(int64_t)b * P.max_blocks + t];
+    const uint16_t* kp = P.kc + (blk * P.G + g) * (int64_t)(MAPS * KT * DK);
+    const uint16_t* vp = P.vc + (blk * P.G + g) * (int64_t)(KT * DV);
+    u16x8 kreg[MAPS][PER_K], vreg[VBLK][4];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+      for (int i = 0; i < PER_K; ++i) kreg[m][i] = load8(kp + m * KT * DK + (int64_t)(tid + 256 * i) * 8);
+#pragma unroll
+    for (int i = 0; i < VBLK; ++i) {
+      const int c = tid + 256 * i;            // block: keys 4 * (c & 15) .. + 3, columns 8 * (c >> 4) .. + 7
+      if (c < 2 * DV) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) vreg[i][kk] = load8(vp + (int64_t)(4 * (c & 15) + kk) * DV + 8 * (c >> 4));
+      }
+    }
+    __syncthreads();   // the previous page's reads are done
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+      for (int i = 0; i < PER_K; ++i) {
+        const int c = tid + 256 * i;
+        const int row = c / NCH_K, ch = c % NCH_K;
+        const int sw = sm_row_swz(row) >> SWS;
+        *reinterpret_cast<u16x8*>(&k_s[m * KT * DK + row * DK + ((ch ^ sw) * 8)]) = kreg[m][i];
+      }
+#pragma unroll
+    for (int i = 0; i < VBLK; ++i) {
+      const int c = tid + 256 * i;
+      if (c < 2 * DV) {
+        const int kb = c & 15, dc = c >> 4;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int row = 8 * dc + e;
+          u16x4 tv;
+          tv[0] = vreg[i][0][e];
+          tv[1] = vreg[i][1][e];
+          tv[2] = vreg[i][2][e];
+          tv[3] = vreg[i][3][e];
+          *reinterpret_cast<u16x4*>(&v_s[row * KT + (((kb >> 1) ^ ((row >> 1) & 7)) * 8) + 4 * (kb & 1)]) = tv;
+        }
+      }
+    }
+    __syncthreads();
+
+    const int kbase = t * KT;
+    const float fd = (float)(qpos - kbase - 8 * h);
+    const bool need_mask = kbase + KT - 1 > wq_lo || (W > 0 && wq_hi - kbase >= W);
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      f32x4 sacc[4];
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau) {
+        const int row = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
+        const int sw = sm_row_swz(row) >> SWS;
+        sacc[tau] = (f32x4)(0.f);
+#pragma unroll
+        for (int s2 = 0; s2 < DS; ++s2) {
+          const int ch = 4 * s2 + h;
+          const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&k_s[m * KT * DK + row * DK + ((ch ^ sw) * 8)]));
+          sacc[tau] = mfma16(a, qf[m][s2], sacc[tau]);
+        }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          float sv = sacc[tau][rr] * P.scale_log2;
+          if (need_mask) {
+            const float d = fd - (float)(32 * (tau >> 1) + 4 * (tau & 1) + rr);
+            sv = (d >= 0.f && d < fW) ? sv : -INFINITY;
+          }
+          sacc[tau][rr] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mnew = fmaxf(mrun[m], mx);
+      const float muse = mnew == -INFINITY ? 0.f : mnew;   // nothing visible yet: weights and factor 0
+      const float corr = __builtin_amdgcn_exp2f(mrun[m] - muse);
+      mrun[m] = mnew;
+      bf16x8 pf[2];
+      float ls = 0.f;
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const float pv = __builtin_amdgcn_exp2f(sacc[tau][rr] - muse);
+          ls += pv;
+          pf[tau >> 1][4 * (tau & 1) + rr] = (__bf16)pv;
+        }
+      ls += __shfl_xor(ls, 16, 64);
+      ls += __shfl_xor(ls, 32, 64);
+      lrun[m] = lrun[m] * corr + ls;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[m][dt] *= corr;
+#pragma unroll
+      for (int gg = 0; gg < 2; ++gg) {
+        const int ch = 4 * gg + h;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const int row = 16 * dt + col;
+          const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&v_s[row * KT + ((ch ^ ((row >> 1) & 7)) * 8)]));
+          o[m][dt] = mfma16(a, pf[gg], o[m][dt]);
+        }
+      }
+    }
+  }
+  // lane (query col, h) holds value columns 16 dt + 4 h + rr of its query
+  float inv[MAPS];
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) inv[m] = 1.0f / lrun[m];
+  float ss = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      float v = o[0][dt][rr] * inv[0];
+      if (MAPS == 2) v -= P.lam * (o[MAPS - 1][dt][rr] * inv[MAPS - 1]);
+      o[0][dt][rr] = v;
+      ss += v * v;
+    }
+  float rs = 1.0f;
+  if (P.unit_eps >= 0.f) {
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    rs = P.out_scale / sqrtf(ss / (float)DV + P.unit_eps);
+  }
+  if (!row_ok) return;
+  if (P.gate) rs *= sigmoidf_(bf2f(P.gate[(int64_t)(q0 + r) * P.g_stride + hq]));
+  uint16_t* op = P.out + (int64_t)(q0 + r) * P.H * DV + (int64_t)hq * DV;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    u16x4 ov;
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) ov[rr] = f2bf(o[0][dt][rr] * rs);
+    *reinterpret_cast<u16x4*>(op + 16 * dt + 4 * h) = ov;
+  }
+}
+
+template <int DK, int DV, int MAPS>
+void launch_sm_mfma_one(const SmMfmaParams& P, dim3 grid, hipStream_t stream) {
+  constexpr size_t smem = (size_t)(MAPS * 64 * DK + DV * 64) * sizeof(uint16_t);
+  static bool attr_set = false;   // more than 64 KB of dynamic LDS needs the attribute once
+  if (smem > 65536 && !attr_set) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&softmax_attention_mfma_kernel<DK, DV, MAPS>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    attr_set = true;
+  }
+  softmax_attention_mfma_kernel<DK, DV, MAPS><<<grid, 256, smem, stream>>>(P);
+}
+
+template <int DK, int MAPS>
+bool launch_sm_mfma_dv(const SmMfmaParams& P, int dv, dim3 grid, hipStream_t stream) {
+  switch (dv) {
+    case 32: launch_sm_mfma_one<DK, 32, MAPS>(P, grid, stream); return true;
+    case 64: launch_sm_mfma_one<DK, 64, MAPS>(P, grid, stream); return true;
+    case 128: launch_sm_mfma_one<DK, 128, MAPS>(P, grid, stream); return true;
+    case 256:
+      if (MAPS == 1) {
+        launch_sm_mfma_one<DK, 256, 1>(P, grid, stream);
+        return true;
+      }
+      return false;
+    default: return false;
+  }
+}
+
+template <int MAPS>
+bool launch_sm_mfma_dk(const SmMfmaParams& P, int dk, int dv, dim3 grid, hipStream_t stream) {
+  switch (dk) {
+    case 32: return launch_sm_mfma_dv<32, MAPS>(P, dv, grid, stream);
+    case 64: return launch_sm_mfma_dv<64, MAPS>(P, dv, grid, stream);
+    case 128: return launch_sm_mfma_dv<128, MAPS>(P, dv, grid, stream);
+    case 256: return MAPS == 1 ? launch_sm_mfma_dv<256, 1>(P, dv, grid, stream) : false;
+    default: return false;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// MFMA form for single-token rows (bf16): the columns of the 16-wide tiles are the heads that
+// share one KV head, so a page is read once for the whole group (and once for both maps of a
+// head: they share V). Workgroup = 4 waves = (part, KV head, token row); the row's visible pages
+// are dealt round-robin to the 4 * parts waves of the row. K fragments go from the page straight
+// into the MFMA A operand; V is transposed through a wave-private LDS tile (V^T [DV][64], as in
+// the prompt kernel). Every wave keeps its own running (max, sum, accumulator) per head and map
+// and writes them as one partial; softmax_decode_reduce merges the partials of a (row, head) in a
+// fixed order, combines the maps, normalises, gates and writes bf16.
+//
+// ws: fp32 [T, H, MAPS, 4 * parts, DV + 4]  (accumulator, then max (log2 domain), sum, 2 unused)
+template <int DK, int DV, int MAPS>
+__global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
+    float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
+    const uint16_t* __restrict__ vc, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ pos, int H, int G, float scale_log2, int window) {
+  constexpr int KT = 64;
+  constexpr int DS = DK / 32;
+  constexpr int DT = DV / 16;
+  constexpr int VBLK = DV / 32;   // (4 keys x 8 columns) blocks per lane per page
+  extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
+  const int part = blockIdx.x, parts = gridDim.x, g = blockIdx.y;
+  const int64_t row = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  uint16_t* v_s = sm_lds + w * (DV * KT);
+  const int col = lane & 15, h = lane >> 4;
+  const int grp = H / G;
+  const int head = g * grp + (col < grp ? col : grp - 1);
+  const int i = pos[row];
+  const int lo = window > 0 && i - window + 1 > 0 ? i - window + 1 : 0;
+  const int p_lo = lo / KT, p_hi = i / KT;           // i < 0: no pages
+  const int n_pages = i < 0 ? 0 : p_hi - p_lo + 1;
+  const int stride = 4 * parts;
+  const int n_it = (n_pages + stride - 1) / stride;  // the same for all four waves (barriers inside)
+  const int32_t* bt = block_tables + (int64_t)tok_seq[row] * max_blocks;
+
+  bf16x8 qf[MAPS][DS];
+  {
+    const uint16_t* qp = q + row * q_stride + (int64_t)head * MAPS * DK;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+      for (int s2 = 0; s2 < DS; ++s2) qf[m][s2] = as_bf16x8(load8(qp + m * DK + 32 * s2 + 8 * h));
+  }
+  f32x4 o[MAPS][DT];
+  float mrun[MAPS], lrun[MAPS];
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) {
+    mrun[m] = -INFINITY;
+    lrun[m] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[m][dt] = (f32x4)(0.f);
+  }
+
+  for (int it = 0; it < n_it; ++it) {
+    const int pg = p_lo + it * stride + part * 4 + w;
+    const bool have = pg <= p_hi;
+    const int64_t blk = have ? bt[pg] : 0;
+    const uint16_t* kp = kc + (blk * G + g) * (int64_t)(MAPS * KT * DK);
+    const uint16_t* vp = vc + (blk * G + g) * (int64_t)(KT * DV);
+    __syncthreads();   // the previous page's reads of this wave's tile are done
+    if (have) {
+#pragma unroll
+      for (int bi = 0; bi < VBLK; ++bi) {
+        const int c = lane + 64 * bi;            // block: keys 4 * (c & 15) .. + 3, columns 8 * (c >> 4) .. + 7
+        const int kb = c & 15, dc = c >> 4;
+        u16x8 vreg[4];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) vreg[kk] = load8(vp + (int64_t)(4 * kb + kk) * DV + 8 * dc);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int r = 8 * dc + e;
+          u16x4 tv;
+          tv[0] = vreg[0][e];
+          tv[1] = vreg[1][e];
+          tv[2] = vreg[2][e];
+          tv[3] = vreg[3][e];
+          *reinterpret_cast<u16x4*>(&v_s[r * KT + (((kb >> 1) ^ ((r >> 1) & 7)) * 8) + 4 * (kb & 1)]) = tv;
+        }
+      }
+    }
+    __syncthreads();
+    if (!have) continue;
+    const int kbase = pg * KT;
+    const bool need_mask = kbase < lo || kbase + KT - 1 > i;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      f32x4 sacc[4];
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau) {
+        const int kr = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
+        sacc[tau] = (f32x4)(0.f);
+#pragma unroll
+        for (int s2 = 0; s2 < DS; ++s2) {
+          const bf16x8 a = as_bf16x8(load8(kp + m * KT * DK + kr * DK + 32 * s2 + 8 * h));
+          sacc[tau] = mfma16(a, qf[m][s2], sacc[tau]);
+        }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          float sv = sacc[tau][rr] * scale_log2;
+          if (need_mask) {
+            const int j = kbase + 32 * (tau >> 1) + 8 * h + 4 * (tau & 1) + rr;
+            sv = (j >= lo && j <= i) ? sv : -INFINITY;
+          }
+          sacc[tau][rr] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mnew = fmaxf(mrun[m], mx);     // every visited page holds a visible key
+      const float corr = __builtin_amdgcn_exp2f(mrun[m] - mnew);
+      mrun[m] = mnew;
+      bf16x8 pf[2];
+      float ls = 0.f;
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const float pv = __builtin_amdgcn_exp2f(sacc[tau][rr] - mnew);
+          ls += pv;
+          pf[tau >> 1][4 * (tau & 1) + rr] = (__bf16)pv;
+        }
+      ls += __shfl_xor(ls, 16, 64);
+      ls += __shfl_xor(ls, 32, 64);
+      lrun[m] = lrun[m] * corr + ls;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[m][dt] *= corr;
+#pragma unroll
+      for (int gg = 0; gg < 2; ++gg) {
+        const int ch = 4 * gg + h;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const int r = 16 * dt + col;
+          const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&v_s[r * KT + ((ch ^ ((r >> 1) & 7)) * 8)]));
+          o[m][dt] = mfma16(a, pf[gg], o[m][dt]);
+        }
+      }
+    }
+  }
+  if (col >= grp) return;
+  const int slot = part * 4 + w;
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) {
+    float* wp = ws + ((((int64_t)row * H + head) * MAPS + m) * stride + slot) * (DV + 4);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(wp + 16 * dt + 4 * h) = o[m][dt];
+    if (h == 0) {
+      wp[DV] = mrun[m];
+      wp[DV + 1] = lrun[m];
+    }
+  }
+}
+
+// one wave per (token row, head): merge the partials of each map, a_0 - lam * a_1, unit RMS, gate
+__global__ void __launch_bounds__(64) softmax_decode_reduce_kernel(
+    uint16_t* __restrict__ out, const float* __restrict__ ws, int slots, const uint16_t* __restrict__ gate,
+    int64_t g_stride, int H, int dv, int maps, float lam, float unit_eps, float out_scale) {
+  const int64_t row = blockIdx.x;
+  const int head = blockIdx.y, lane = threadIdx.x;
+  constexpr int MAXV = 4;   // dv <= 256
+  float res[MAXV] = {0.f, 0.f, 0.f, 0.f};
+  for (int m = 0; m < maps; ++m) {
+    const float* wp = ws + (((int64_t)row * H + head) * maps + m) * slots * (int64_t)(dv + 4);
+    float M = -INFINITY;
+    for (int s = 0; s < slots; ++s) M = fmaxf(M, wp[(int64_t)s * (dv + 4) + dv]);
+    float L = 0.f, acc[MAXV] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < slots; ++s) {
+      const float* sp = wp + (int64_t)s * (dv + 4);
+      const float ms = sp[dv];
+      if (ms == -INFINITY) continue;   // a wave that got no page
+      const float f = __builtin_amdgcn_exp2f(ms - M);
+      L += sp[dv + 1] * f;
+#pragma unroll
+      for (int u = 0; u < MAXV; ++u)
+        if (lane + 64 * u < dv) acc[u] += sp[lane + 64 * u] * f;
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;   // padding row: zeros
+#pragma unroll
+    for (int u = 0; u < MAXV; ++u) res[u] = m == 0 ? acc[u] * inv : res[u] - lam * (acc[u] * inv);
+  }
+  float r = 1.0f;
+  if (unit_eps >= 0.f) {
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < MAXV; ++u)
+      if (lane + 64 * u < dv) ss += res[u] * res[u];
+    ss = wave_sum(ss);
+    r = out_scale / sqrtf(ss / (float)dv + unit_eps);
+  }
+  if (gate) r *= sigmoidf_(bf2f(gate[row * g_stride + head]));
+#pragma unroll
+  for (int u = 0; u < MAXV; ++u)
+    if (lane + 64 * u < dv) out[(row * H + head) * (int64_t)dv + lane + 64 * u] = f2bf(res[u] * r);
+}
+
+template <int DK, int DV, int MAPS>
+void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
+                          const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos,
+                          int H, int G, float scale_log2, int window, dim3 grid, hipStream_t stream) {
+  constexpr size_t smem = (size_t)4 * DV * 64 * sizeof(uint16_t);
+  static bool attr_set = false;
+  if (smem > 65536 && !attr_set) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&softmax_decode_mfma_kernel<DK, DV, MAPS>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    attr_set = true;
+  }
+  softmax_decode_mfma_kernel<DK, DV, MAPS><<<grid, 256, smem, stream>>>(ws, q, q_stride, kc, vc, block_tables,
+                                                                       max_blocks, tok_seq, pos, H, G, scale_log2,
+                                                                       window);
+}
+
+#define NGA_SM_DEC_ARGS ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, grid, stream
+template <int DK, int MAPS>
+bool launch_sm_decode_dv(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
+                         const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos, int H,
+                         int G, float scale_log2, int window, int dv, dim3 grid, hipStream_t stream) {
+  switch (dv) {
+    case 32: launch_sm_decode_one<DK, 32, MAPS>(NGA_SM_DEC_ARGS); return true;
+    case 64: launch_sm_decode_one<DK, 64, MAPS>(NGA_SM_DEC_ARGS); return true;
+    case 128: launch_sm_decode_one<DK, 128, MAPS>(NGA_SM_DEC_ARGS); return true;
+    case 256:
+      if (MAPS == 1) {
+        launch_sm_decode_one<DK, 256, 1>(NGA_SM_DEC_ARGS);
+        return true;
+      }
+      return false;
+    default: return false;
+  }
+}
+
+template <int MAPS>
+bool launch_sm_decode_dk(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
+                         const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos, int H,
+                         int G, float scale_log2, int window, int dk, int dv, dim3 grid, hipStream_t stream) {
+#define NGA_SM_DEC_DV(DKV) launch_sm_decode_dv<DKV, MAPS>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, dv, grid, stream)
+  switch (dk) {
+    case 32: return NGA_SM_DEC_DV(32);
+    case 64: return NGA_SM_DEC_DV(64);
+    case 128: return NGA_SM_DEC_DV(128);
+    case 256: return MAPS == 1 ? launch_sm_decode_dv<256, 1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G, scale_log2, window, dv, grid, stream) : false;
+    default: return false;
+  }
+#undef NGA_SM_DEC_DV
+}
+#undef NGA_SM_DEC_ARGS
+
 }  // namespace
+
+// Parts (workgroups per row and KV head) of the single-token MFMA kernel: enough waves to fill
+// the chip, never more than the pages a row can see. Fixed by sizes the host knows, so a
+// captured step keeps its launch shape.
+int softmax_decode_parts(int rows, int G, int max_ctx, int window) {
+  const int64_t span = window > 0 && window < max_ctx ? window : max_ctx;
+  const int pages = (int)(span / 64) + 2;
+  const int by_pages = (pages + 3) / 4;
+  const int target = 8192;   // waves to launch: 8 per SIMD on 256 CUs
+  const int by_fill = (target + rows * G * 4 - 1) / (rows * G * 4);
+  const int p = by_pages < by_fill ? by_pages : by_fill;
+  return p < 1 ? 1 : (p > 32 ? 32 : p);
+}
+
+// ws: fp32 [T, H, maps, 4 * parts, dv + 4]
+void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
+                                const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
+                                const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
+                                const int32_t* pos, int64_t T, int H, int G, int dk, int dv, float scale, int window,
+                                int maps, float lam, float unit_eps, float out_scale, hipStream_t stream) {
+  if (T == 0) return;
+  const dim3 grid((unsigned)parts, (unsigned)G, (unsigned)T);
+  const float scale_log2 = scale * 1.4426950408889634f;
+  const bool ok = maps == 2 ? launch_sm_decode_dk<2>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
+                                                     scale_log2, window, dk, dv, grid, stream)
+                            : launch_sm_decode_dk<1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
+                                                     scale_log2, window, dk, dv, grid, stream);
+  if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
+  softmax_decode_reduce_kernel<<<dim3((unsigned)T, (unsigned)H), 64, 0, stream>>>(out, ws, 4 * parts, gate, g_stride, H,
+                                                                                   dv, maps, lam, unit_eps, out_scale);
+}
+
+// Head sizes of the MFMA forms: dk, dv in {32, 64, 128} (one map: also 256); at most 16 heads per
+// KV head (the columns of one tile in the single-token kernel).
+bool softmax_attention_mfma_supported(int dk, int dv, int group, int maps) {
+  auto ok = [&](int d) { return d == 32 || d == 64 || d == 128 || (maps == 1 && d == 256); };
+  return (maps == 1 || maps == 2) && ok(dk) && ok(dv) && group >= 1 && group <= 16;
+}
+
+// prompt portions: sequence b owns rows [cu_q[b], cu_q[b + 1]) of q / gate / out, the last ones of
+// its ctx_lens[b] keys. q rows must be 16-byte aligned (checked by the caller).
+void launch_softmax_attention_mfma(uint16_t* out, const uint16_t* q, int64_t q_stride, const uint16_t* gate,
+                                   int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
+                                   const int32_t* block_tables, int max_blocks, const int32_t* cu_q,
+                                   const int32_t* ctx_lens, int B, int max_q_len, int H, int G, int dk, int dv,
+                                   float scale, int window, int maps, float lam, float unit_eps, float out_scale,
+                                   hipStream_t stream) {
+  if (B == 0 || max_q_len == 0) return;
+  SmMfmaParams P{out, q, gate, kc, vc, block_tables, cu_q, ctx_lens, q_stride, g_stride, max_blocks, H, G, window,
+                 scale * 1.4426950408889634f, lam, unit_eps, out_scale};
+  const dim3 grid((unsigned)((max_q_len + 63) / 64), (unsigned)H, (unsigned)B);
+  const bool ok = maps == 2 ? launch_sm_mfma_dk<2>(P, dk, dv, grid, stream) : launch_sm_mfma_dk<1>(P, dk, dv, grid, stream);
+  if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
+}
 
 void launch_headnorm_cache(void* proj, int64_t stride, const int32_t* slots, void* kc, void* vc, int64_t T, int nq,
                            int nk, int dk, int nv, int dv, float eps, const float* qw, const float* kw,

@@ -556,3 +556,44 @@ def test_lambda_of_the_layer():
     f = {k: w["l0.mix." + k].double() for k in ("lq1", "lk1", "lq2", "lk2")}
     want = math.exp(float((f["lq1"] * f["lk1"]).sum())) - math.exp(float((f["lq2"] * f["lk2"]).sum())) + 0.2
     assert abs(m.layers[0]["lam"] - want) < 1e-12
+
+
+@pytest.mark.gpu
+def test_mfma_forms_run_and_agree_with_the_row_kernel():
+    """bf16 rows with tile-sized heads take the MFMA kernels (not the row kernel); at sizes of real
+    layers (long contexts, 128-wide heads, 16 heads per KV head, both maps, a window that starts
+    and ends inside pages) the two forms agree to bf16 rounding."""
+    torch.manual_seed(11)
+    dev = "cuda"
+    qa = torch.zeros(4, 256, dtype=torch.bfloat16, device=dev)
+    assert ops.softmax_attention_mfma_ok(qa, 32, 64, 2, 2) and ops.softmax_attention_mfma_ok(qa, 256, 256, 16, 1)
+    assert not ops.softmax_attention_mfma_ok(qa.float(), 32, 64, 2, 2)
+    assert not ops.softmax_attention_mfma_ok(qa, 48, 64, 2, 2) and not ops.softmax_attention_mfma_ok(qa, 256, 64, 1, 2)
+    for H, G, dk, dv, W, maps in ((8, 2, 128, 128, 0, 2), (16, 1, 128, 128, 300, 1), (4, 1, 256, 256, 1000, 1),
+                                  (2, 2, 64, 128, 77, 2)):
+        ctxs, qlens = [1500, 700, 65], [1500, 130, 1]
+        nb, mb = 40, 24
+        kc = (torch.randn(nb, G * maps, 64, dk, device=dev) * 0.5).bfloat16()
+        vc = torch.randn(nb, G, 64, dv, device=dev).bfloat16()
+        perm = torch.randperm(nb)[:36].tolist()
+        bts = torch.zeros(3, mb, dtype=torch.int32)
+        bts[0, :24] = torch.tensor(perm[:24])
+        bts[1, :11] = torch.tensor(perm[24:35])
+        bts[2, :2] = torch.tensor([perm[35], perm[0]])
+        bts = bts.to(dev)
+        T = sum(qlens)
+        q = torch.randn(T, H * maps * dk, device=dev).bfloat16()
+        gate = torch.randn(T, H, device=dev).bfloat16()
+        cu = torch.tensor([0, 1500, 1630, 1631], dtype=torch.int32, device=dev)
+        cx = torch.tensor(ctxs, dtype=torch.int32, device=dev)
+        seq = torch.tensor([0] * 1500 + [1] * 130 + [2], dtype=torch.int32, device=dev)
+        pos = torch.cat([torch.arange(c - n, c) for c, n in zip(ctxs, qlens)]).int().to(dev)
+        kw = dict(window=W, maps=maps, lam=0.4, unit_eps=1e-5 if maps == 2 else None, out_scale=0.7, gate=gate)
+        want = ops.softmax_attention(q, kc, vc, bts, seq, pos, H, G, dk, dv, dk ** -0.5, **kw).float()
+        got = ops.softmax_attention_prefill(q, kc, vc, bts, cu, cx, 1500, H, G, dk, dv, dk ** -0.5, **kw).float()
+        assert (got - want).abs().max().item() < 0.03 * max(1.0, want.abs().max().item()), ("prompt kernel", H, G, dk, dv, W)
+        pick = torch.tensor([0, 63, 64, 700, 1499, 1500, 1629, 1630], device=dev)
+        kw["gate"] = gate[pick].contiguous()
+        got1 = ops.softmax_attention_rows(q[pick].contiguous(), kc, vc, bts, seq[pick].contiguous(),
+                                          pos[pick].contiguous(), H, G, dk, dv, dk ** -0.5, max_ctx=1536, **kw).float()
+        assert (got1 - want[pick]).abs().max().item() < 0.03 * max(1.0, want.abs().max().item()), ("single-token kernel", H, G, dk, dv, W)
