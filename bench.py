@@ -106,6 +106,8 @@ def parse(argv=None):
                     help="stripe each replica's index over its tp ranks (broadcast + all-gather merge)")
     ap.add_argument("--design-sizes", default=None,
                     help="--workload designs: comma list of s, m, l (benchmarks/design_compare.py)")
+    ap.add_argument("--design-models", default="bidasun",
+                    help="--workload designs: comma list of the designs to run beside Mistral (bidasun, biruvik)")
     ap.add_argument("--workload", choices=("rag", "agent", "designs"), default="rag",
                     help="agent: query-decomposition agent, one TP=N replica + N-way sharded index")
     ap.add_argument("--kv-cache-fraction", type=float, default=None)
@@ -313,8 +315,8 @@ def main(argv=None):
         run_agent(args, world_env, shared)
         return
     if args.workload == "designs":
-        # Bidasun beside the equal-size sliding-window Mistral: engine prefill / decode rates and
-        # the attention kernels against their rooflines (one GPU; the default workload is untouched)
+        # Bidasun / Biruvik beside the equal-size sliding-window Mistral: engine prefill / decode
+        # rates and the mixer kernels against their rooflines (one GPU; the default workload is untouched)
         from benchmarks.design_compare import run as run_designs
 
         run_designs(args)

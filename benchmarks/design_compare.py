@@ -1,8 +1,8 @@
-"""Bidasun beside the closest Llama-layout model (Mistral with a sliding window) at equal sizes:
-prefill and decode throughput through the serving engine, and the attention kernels alone with
-their distance from the roofline. Random weights, synthetic token ids.
+"""The layer-list designs (Bidasun, Biruvik) beside the closest Llama-layout model (Mistral with a
+sliding window) at equal sizes: prefill and decode throughput through the serving engine, and the
+mixer kernels alone with their distance from the roofline. Random weights, synthetic token ids.
 
-    python bench.py --workload designs [--design-sizes s,m,l]
+    python bench.py --workload designs [--design-sizes s,m,l] [--design-models bidasun,biruvik]
 
 Prints one JSON line (``metric: design_compare``); bench.py's default workload is untouched.
 """
@@ -23,13 +23,20 @@ VOCAB = 32768
 PEAK_BF16 = 2.5e15      # dense MFMA flop/s
 PEAK_HBM = 8.0e12       # bytes/s
 PEAK_TRANS = 256 * 16 * 2.4e9   # transcendental lanes/s: 256 CUs x 4 SIMDs x 4 lanes/clk at 2.4 GHz
+PEAK_VALU = 256 * 4 * 16 * 2 * 2.4e9   # fp32 flop/s of the vector ALUs (FMA = 2), unpacked
+BIRUVIK_PATTERN = ("attention", "latent_attention", "hgrn2", "attention")
+BIRUVIK_RANK = 256    # latent size of the latent-attention layers
 
 
 def _engine(kind: str, z: dict, max_len: int, pages: int, seqs: int):
     from nv_genai_amd.engine.llm_engine import EngineConfig, LLMEngine
-    from nv_genai_amd.models.config import LlamaConfig, bidasun_uniform
+    from nv_genai_amd.models.config import LlamaConfig, bidasun_uniform, biruvik_layers
 
-    if kind == "bidasun":
+    if kind == "biruvik":
+        pat = [BIRUVIK_PATTERN[i % len(BIRUVIK_PATTERN)] for i in range(z["layers"])]
+        mcfg = biruvik_layers(pat, z["hidden"], z["heads"], z["kv"], z["d"], z["d"], z["ffn"], window=z["window"],
+                              kv_rank=BIRUVIK_RANK, vocab_size=VOCAB)
+    elif kind == "bidasun":
         mcfg = bidasun_uniform(z["layers"], z["hidden"], z["heads"], z["kv"], z["d"], z["d"], z["ffn"], z["window"], 4,
                                vocab_size=VOCAB, max_position=max_len)
     else:
@@ -142,17 +149,106 @@ def kernel_times(z: dict, iters: int = 20) -> dict:
     return out
 
 
+def biruvik_kernel_times(z: dict, iters: int = 20) -> dict:
+    """The Biruvik mixer kernels alone on one layer's shapes beside the softmax kernels of the
+    Llama layout: differential attention (two maps, causal) against causal softmax attention,
+    windowed latent attention (multi-query over the latent page) against windowed softmax
+    attention, and the HGRN2 scan (no counterpart: priced against the fp32 vector rate for prompts
+    and against the HBM bytes of the state for single rows)."""
+    from nv_genai_amd import ops
+
+    dev, bf = "cuda", torch.bfloat16
+    H, G, D, W, R = z["heads"], z["kv"], z["d"], z["window"], BIRUVIK_RANK
+    nb, L = z["pf"]
+    nd, ctx = z["dec"]
+    pages_seq = -(-max(L, ctx) // 64)
+    nseq = max(nb, nd)
+    npg = nseq * pages_seq
+    bt = torch.arange(npg, dtype=torch.int32, device=dev).view(nseq, pages_seq)
+    k2 = (torch.randn(npg, 2 * G, 64, D, device=dev) * 0.5).to(bf)      # both maps
+    vr = (torch.randn(npg, G, 64, D, device=dev) * 0.5).to(bf)          # row-major values
+    cc = (torch.randn(npg, 1, 64, R, device=dev) * 0.5).to(bf)          # latent pages
+    kl = k2[:, :G].contiguous()
+    vt = vr.transpose(2, 3).contiguous()                               # V^T pages of the Llama layout
+    T = nb * L
+    cu = torch.arange(0, T + 1, L, dtype=torch.int32, device=dev)
+    cx = torch.full((nb,), L, dtype=torch.int32, device=dev)
+    out = {}
+    # ---- prompt portions
+    q2 = torch.randn(T, H * 2 * D, device=dev).to(bf)
+    q1 = q2[:, :H * D].contiguous()
+    ql = torch.randn(T, H * R, device=dev).to(bf)
+    gate = torch.randn(T, H, device=dev).to(bf)
+    pairs_c = nb * (L * (L + 1) // 2) * H
+    pairs_w = nb * sum(min(i + 1, W) for i in range(L)) * H
+    t_diff = _timed(lambda: ops.softmax_attention_prefill(q2, k2, vr, bt, cu, cx, L, H, G, D, D, D ** -0.5, maps=2,
+                                                          lam=0.4, unit_eps=1e-5, out_scale=0.7), iters)
+    t_soft_c = _timed(lambda: ops.prefill_attention_paged(q1, kl, vt, bt, cu, cx, H, G, D, L, D ** -0.5, window=0, impl=4),
+                      iters)
+    t_lat = _timed(lambda: ops.softmax_attention_prefill(ql, cc, cc, bt, cu, cx, L, H, 1, R, R, D ** -0.5, window=W,
+                                                         gate=gate), iters)
+    t_soft_w = _timed(lambda: ops.prefill_attention_paged(q1, kl, vt, bt, cu, cx, H, G, D, L, D ** -0.5, window=W, impl=4),
+                      iters)
+    out["prefill"] = {
+        "differential_ms": round(t_diff * 1e3, 3), "softmax_causal_ms": round(t_soft_c * 1e3, 3),
+        "differential_mfma_frac": round(2 * 4.0 * pairs_c * D / t_diff / PEAK_BF16, 4),
+        "softmax_causal_mfma_frac": round(4.0 * pairs_c * D / t_soft_c / PEAK_BF16, 4),
+        "latent_ms": round(t_lat * 1e3, 3), "softmax_window_ms": round(t_soft_w * 1e3, 3),
+        "latent_mfma_frac": round(4.0 * pairs_w * R / t_lat / PEAK_BF16, 4),
+        "softmax_window_mfma_frac": round(4.0 * pairs_w * D / t_soft_w / PEAK_BF16, 4)}
+    # ---- single-token rows
+    seq = torch.arange(nd, dtype=torch.int32, device=dev)
+    pos = torch.full((nd,), ctx - 1, dtype=torch.int32, device=dev)
+    cxd = torch.full((nd,), ctx, dtype=torch.int32, device=dev)
+    ws = ops.DecodeWorkspace(nd, H, G, ctx, dev, None, D=D)
+    t_diffd = _timed(lambda: ops.softmax_attention_rows(q2[:nd], k2, vr, bt, seq, pos, H, G, D, D, D ** -0.5, max_ctx=ctx,
+                                                        maps=2, lam=0.4, unit_eps=1e-5, out_scale=0.7), iters)
+    t_softd_c = _timed(lambda: ops.decode_attention(q1[:nd], kl, vt, bt, cxd, H, G, ctx, D ** -0.5, ws=ws, window=0), iters)
+    t_latd = _timed(lambda: ops.softmax_attention_rows(ql[:nd], cc, cc, bt, seq, pos, H, 1, R, R, D ** -0.5, max_ctx=ctx,
+                                                       window=W, gate=gate[:nd]), iters)
+    t_softd_w = _timed(lambda: ops.decode_attention(q1[:nd], kl, vt, bt, cxd, H, G, ctx, D ** -0.5, ws=ws, window=W), iters)
+    vis = min(ctx, W)
+    out["decode"] = {
+        "differential_ms": round(t_diffd * 1e3, 4), "softmax_causal_ms": round(t_softd_c * 1e3, 4),
+        "differential_hbm_frac": round(nd * G * ctx * 3 * D * 2.0 / t_diffd / PEAK_HBM, 4),
+        "softmax_causal_hbm_frac": round(nd * G * ctx * 2 * D * 2.0 / t_softd_c / PEAK_HBM, 4),
+        "latent_ms": round(t_latd * 1e3, 4), "softmax_window_ms": round(t_softd_w * 1e3, 4),
+        "latent_hbm_frac": round(nd * vis * R * 2.0 / t_latd / PEAK_HBM, 4),
+        "softmax_window_hbm_frac": round(nd * G * vis * 2 * D * 2.0 / t_softd_w / PEAK_HBM, 4)}
+    # ---- HGRN2 scan: prompts of L rows, then one row per sequence
+    proj = torch.randn(T, 3 * H * D, device=dev).to(bf)
+    fb = torch.zeros(H * D, device=dev)
+    low = torch.full((H * D,), 0.3, device=dev)
+    state = torch.zeros(nseq, H, D, D, device=dev)
+    slots_p = torch.arange(nb, dtype=torch.int32, device=dev)
+    pos_p = torch.arange(L, dtype=torch.int32, device=dev).repeat(nb)
+    t_scan = _timed(lambda: ops.hgrn2_scan(proj, fb, low, state, H, D, D, cu, slots_p, pos_p), max(2, iters // 4))
+    t_scand = _timed(lambda: ops.hgrn2_scan(proj[:nd], fb, low, state, H, D, D, None, seq, pos), iters)
+    out["hgrn2"] = {"prefill_ms": round(t_scan * 1e3, 3), "prefill_tok_s": round(T / t_scan),
+                    "prefill_valu_frac": round(6.0 * T * H * D * D / t_scan / PEAK_VALU, 4),
+                    "decode_ms": round(t_scand * 1e3, 4),
+                    "decode_hbm_frac": round(nd * H * D * D * 4 * 2.0 / t_scand / PEAK_HBM, 4)}
+    return out
+
+
 def run(args) -> None:
     names = [s for s in (args.design_sizes or "s,m,l").split(",") if s]
+    models = [m for m in (getattr(args, "design_models", None) or "bidasun").split(",") if m]
+    if any(m not in ("bidasun", "biruvik") for m in models):
+        raise SystemExit(f"--design-models: unknown design in {models} (bidasun, biruvik)")
     res = {}
     for n in names:
         z = SIZES[n]
         res[n] = {"shape": {k: v for k, v in z.items()}}
-        for kind in ("bidasun", "mistral"):
+        for kind in models + ["mistral"]:
             res[n][kind] = engine_rates(kind, z, max(1, args.steps), max(1, args.warmup))
             torch.cuda.empty_cache()
-        res[n]["attention_kernels"] = kernel_times(z)
-        torch.cuda.empty_cache()
+        if "bidasun" in models:
+            res[n]["attention_kernels"] = kernel_times(z)
+            torch.cuda.empty_cache()
+        if "biruvik" in models:
+            res[n]["biruvik_kernels"] = biruvik_kernel_times(z)
+            torch.cuda.empty_cache()
         print(f"[designs] {n}: {json.dumps(res[n])}", flush=True)
     line = {"metric": "design_compare", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "dtype": "bf16", "data": "synthetic token ids, random weights", "sizes": res}

@@ -5,11 +5,13 @@
 //                f = lower + (1 - lower) * sigmoid(f_pre + f_bias) formed in fp32 in the kernel.
 //
 // A workgroup owns (segment, head, tile of VT value columns): thread (rg, j) keeps the state
-// elements S[rg + RG * k][j] in registers for the whole segment, so the state is read from its
-// slot once and written back once. Rows are staged through LDS TC at a time (activations
-// applied while staging); per row every thread updates its NR state elements and adds its part of
-// o, the RG parts are summed through LDS for all TC rows at once. State, gates and sums are fp32
-// whatever the activation type.
+// elements S[rg * NR + k][j] in registers for the whole segment, so the state is read from its
+// slot once and written back once. Rows are staged through LDS TC at a time: the raw values of the
+// next TC rows are loaded into registers before the current ones are processed, and the
+// activations are applied on the way into LDS. Per row every thread reads its NR gates and
+// queries as 16-byte LDS vectors, updates its NR state elements and adds its part of o; the RG
+// parts are summed through LDS for all TC rows at once. The tile width VT is chosen by the host so
+// that a launch has enough workgroups. State, gates and sums are fp32 whatever the activation type.
 #include "common.h"
 #include "kernels.h"
 
@@ -21,22 +23,25 @@ template <typename T> __device__ __forceinline__ float ldf(const T* p);
 template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf2f(*p); }
 template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
 
-constexpr int TC = 8;   // rows staged per pass
+constexpr int TC = 16;   // rows staged per pass
 
 // proj row: [q_pre (H*d) | f_pre (H*d) | v (H*dv) | ...]. cu == nullptr: segment b is row b.
-template <typename T, int NR>
+// Rows of a head are padded to DP = RG * NR in LDS (q = 0, f = 1: a padded state row stays 0).
+template <typename T, int NR, int VT>
 __global__ void __launch_bounds__(256) hgrn2_scan_kernel(float* __restrict__ out, const T* __restrict__ proj,
                                                          int64_t stride, const float* __restrict__ f_bias,
                                                          const float* __restrict__ lower, float* __restrict__ state,
                                                          int H, int d, int dv, const int32_t* __restrict__ cu,
                                                          const int32_t* __restrict__ slots,
-                                                         const int32_t* __restrict__ pos, int VT) {
-  extern __shared__ float smem[];
-  const int RG = 256 / VT;
-  float* qs = smem;                  // [TC][d]
-  float* fs = qs + TC * d;           // [TC][d]
-  float* vs = fs + TC * d;           // [TC][VT]
-  float* part = vs + TC * VT;        // [TC][RG][VT] = [TC][256]
+                                                         const int32_t* __restrict__ pos) {
+  constexpr int RG = 256 / VT;
+  constexpr int DP = RG * NR;              // padded rows of a head
+  constexpr int NQ = TC * DP / 256;        // q (and f) elements a thread stages per pass
+  constexpr int NV = (TC * VT + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float qs[TC * DP];
+  __shared__ __attribute__((aligned(16))) float fs[TC * DP];
+  __shared__ float vs[TC * VT];
+  __shared__ float part[TC * 256];
   const int vt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t0 = cu ? cu[b] : b, t1 = cu ? cu[b + 1] : b + 1;
   if (t1 <= t0) return;
@@ -50,90 +55,134 @@ __global__ void __launch_bounds__(256) hgrn2_scan_kernel(float* __restrict__ out
   float S[NR];
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
-    const int i = rg + RG * k;
+    const int i = rg * NR + k;
     S[k] = (!fresh && colok && i < d) ? sp[(int64_t)i * dv + col] : 0.f;
   }
   const int qoff = h * d, foff = H * d + h * d, voff = 2 * H * d + h * dv + vt * VT;
+  float rq[NQ], rf[NQ], rv[NV];
+  // raw values of rows [tc, tc + TC) into registers (rows past t1 and padded columns: neutral)
+  auto fetch = [&](int tc) {
+#pragma unroll
+    for (int x = 0; x < NQ; ++x) {
+      const int e = tid + 256 * x, tt = e / DP, i = e % DP;
+      const bool ok = tc + tt < t1 && i < d;
+      const T* pr = proj + (int64_t)(tc + tt) * stride;
+      rq[x] = ok ? ldf(pr + qoff + i) : 0.f;
+      rf[x] = ok ? ldf(pr + foff + i) : 0.f;
+    }
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = tid + 256 * x, tt = e / VT, jj = e % VT;
+      rv[x] = (e < TC * VT && tc + tt < t1 && vt * VT + jj < dv) ? ldf(proj + (int64_t)(tc + tt) * stride + voff + jj) : 0.f;
+    }
+  };
+  fetch(t0);
   for (int tc = t0; tc < t1; tc += TC) {
     const int nt = t1 - tc < TC ? t1 - tc : TC;
-    for (int e = tid; e < nt * d; e += 256) {
-      const int tt = e / d, i = e - tt * d;
-      const T* pr = proj + (int64_t)(tc + tt) * stride;
-      const float qv = ldf(pr + qoff + i);
-      qs[e] = qv / (1.0f + expf(-qv));
-      const float lw = lower[qoff + i];
-      const float fv = ldf(pr + foff + i) + f_bias[qoff + i];
-      fs[e] = lw + (1.0f - lw) * (1.0f / (1.0f + expf(-fv)));
+    __syncthreads();   // the previous pass is done with qs / fs / vs / part
+#pragma unroll
+    for (int x = 0; x < NQ; ++x) {
+      const int e = tid + 256 * x, i = e % DP;
+      if (i < d) {
+        const float lw = lower[qoff + i];
+        qs[e] = rq[x] / (1.0f + expf(-rq[x]));
+        fs[e] = lw + (1.0f - lw) * (1.0f / (1.0f + expf(-(rf[x] + f_bias[qoff + i]))));
+      } else {
+        qs[e] = 0.f;
+        fs[e] = 1.f;
+      }
     }
-    for (int e = tid; e < nt * VT; e += 256) {
-      const int tt = e / VT, jj = e - tt * VT;
-      vs[e] = vt * VT + jj < dv ? ldf(proj + (int64_t)(tc + tt) * stride + voff + jj) : 0.f;
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = tid + 256 * x;
+      if (e < TC * VT) vs[e] = rv[x];
     }
     __syncthreads();
+    if (tc + TC < t1) fetch(tc + TC);   // lands while this pass computes
     for (int tt = 0; tt < nt; ++tt) {
       const float vv = vs[tt * VT + j];
-      const float* fr = fs + tt * d;
-      const float* qr = qs + tt * d;
+      const float4* fr = reinterpret_cast<const float4*>(fs + tt * DP + rg * NR);
+      const float4* qr = reinterpret_cast<const float4*>(qs + tt * DP + rg * NR);
       float p = 0.f;
 #pragma unroll
-      for (int k = 0; k < NR; ++k) {
-        const int i = rg + RG * k;
-        if (i < d) {
-          const float f = fr[i];
-          S[k] = f * S[k] + (1.0f - f) * vv;
-          p += S[k] * qr[i];
+      for (int k4 = 0; k4 < NR / 4; ++k4) {
+        const float4 f4 = fr[k4], q4 = qr[k4];
+        const float fa[4] = {f4.x, f4.y, f4.z, f4.w}, qa[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int k = 4 * k4 + u;
+          S[k] = fa[u] * S[k] + (1.0f - fa[u]) * vv;
+          p += S[k] * qa[u];
         }
       }
       part[tt * 256 + tid] = p;
     }
     __syncthreads();
     for (int e = tid; e < nt * VT; e += 256) {
-      const int tt = e / VT, jj = e - tt * VT;
+      const int tt = e / VT, jj = e % VT;
       if (vt * VT + jj < dv) {
-        float s = 0.f;
-        for (int r = 0; r < RG; ++r) s += part[tt * 256 + r * VT + jj];
-        out[(int64_t)(tc + tt) * H * dv + h * dv + vt * VT + jj] = s;
+        float s2 = 0.f;
+#pragma unroll
+        for (int r = 0; r < RG; ++r) s2 += part[tt * 256 + r * VT + jj];
+        out[(int64_t)(tc + tt) * H * dv + h * dv + vt * VT + jj] = s2;
       }
     }
-    __syncthreads();
   }
   if (sp && colok) {
 #pragma unroll
     for (int k = 0; k < NR; ++k) {
-      const int i = rg + RG * k;
+      const int i = rg * NR + k;
       if (i < d) sp[(int64_t)i * dv + col] = S[k];
     }
   }
 }
 
-template <typename T>
-bool launch_hgrn2_t(float* out, const T* proj, int64_t stride, const float* f_bias, const float* lower, float* state,
-                    int H, int d, int dv, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg,
-                    hipStream_t stream) {
-  const int VT = dv >= 64 ? 64 : (dv >= 32 ? 32 : 16);
-  const int RG = 256 / VT;
+template <typename T, int VT>
+bool launch_hgrn2_vt(float* out, const T* proj, int64_t stride, const float* f_bias, const float* lower, float* state,
+                     int H, int d, int dv, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg,
+                     hipStream_t stream) {
+  constexpr int RG = 256 / VT;
   const int nr = (d + RG - 1) / RG;
   const dim3 grid((unsigned)((dv + VT - 1) / VT), (unsigned)H, (unsigned)n_seg);
-  const size_t smem = (size_t)TC * (2 * d + VT + 256) * sizeof(float);
-#define NGA_HGRN2_CASE(N)                                                                                             \
-  if (nr <= N) {                                                                                                      \
-    hgrn2_scan_kernel<T, N><<<grid, 256, smem, stream>>>(out, proj, stride, f_bias, lower, state, H, d, dv, cu, slots, \
-                                                         pos, VT);                                                    \
-    return true;                                                                                                      \
+#define NGA_HGRN2_CASE(N)                                                                                            \
+  if (nr <= N) {                                                                                                     \
+    hgrn2_scan_kernel<T, N, VT><<<grid, 256, 0, stream>>>(out, proj, stride, f_bias, lower, state, H, d, dv, cu, slots, \
+                                                          pos);                                                      \
+    return true;                                                                                                     \
   }
-  NGA_HGRN2_CASE(2)
+  // at most 256 padded rows per head in LDS: NR <= 64 / 32 / 16 for tiles of 64 / 32 / 16 columns
   NGA_HGRN2_CASE(4)
   NGA_HGRN2_CASE(8)
   NGA_HGRN2_CASE(16)
-  NGA_HGRN2_CASE(32)
-  NGA_HGRN2_CASE(64)
+  if constexpr (VT >= 32) {
+    NGA_HGRN2_CASE(32)
+  }
+  if constexpr (VT >= 64) {
+    NGA_HGRN2_CASE(64)
+  }
 #undef NGA_HGRN2_CASE
   return false;
 }
 
+// The widest value tile that still gives about four workgroups per CU; narrower tiles when the
+// key size needs more row groups than a wide tile leaves.
+template <typename T>
+bool launch_hgrn2_t(float* out, const T* proj, int64_t stride, const float* f_bias, const float* lower, float* state,
+                    int H, int d, int dv, const int32_t* cu, const int32_t* slots, const int32_t* pos, int n_seg,
+                    hipStream_t stream) {
+  const int64_t base = (int64_t)n_seg * H;
+  int vt = dv <= 16 ? 16 : (dv <= 32 ? 32 : 64);
+  while (vt > 16 && base * ((dv + vt - 1) / vt) < 1024) vt /= 2;
+#define NGA_HGRN2_ARGS out, proj, stride, f_bias, lower, state, H, d, dv, cu, slots, pos, n_seg, stream
+  if (vt == 64 && launch_hgrn2_vt<T, 64>(NGA_HGRN2_ARGS)) return true;
+  if (vt >= 32 && launch_hgrn2_vt<T, 32>(NGA_HGRN2_ARGS)) return true;
+  return launch_hgrn2_vt<T, 16>(NGA_HGRN2_ARGS);
+#undef NGA_HGRN2_ARGS
+}
+
 }  // namespace
 
-int hgrn2_max_dim(int dv) { return 64 * (256 / (dv >= 64 ? 64 : (dv >= 32 ? 32 : 16))); }
+int hgrn2_max_dim(int dv) { return 256; }   // padded rows of a head that fit the LDS staging
 
 bool launch_hgrn2_scan(float* out, const void* proj, int64_t stride, const float* f_bias, const float* lower,
                        float* state, int H, int d, int dv, const int32_t* cu, const int32_t* slots, const int32_t* pos,

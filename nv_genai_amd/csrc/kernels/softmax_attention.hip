@@ -460,8 +460,8 @@ bool launch_sm_mfma_dk(const SmMfmaParams& P, int dk, int dv, dim3 grid, hipStre
 
 // ---------------------------------------------------------------------------------------------
 // MFMA form for single-token rows (bf16): the columns of the 16-wide tiles are the heads that
-// share one KV head, so a page is read once for the whole group (and once for both maps of a
-// head: they share V). Workgroup = 4 waves = (part, KV head, token row); the row's visible pages
+// share one KV head (16 per workgroup), so a page is read once for the whole group (and once for
+// both maps of a head: they share V). Workgroup = 4 waves = (part, KV head, token row); the row's visible pages
 // are dealt round-robin to the 4 * parts waves of the row. K fragments go from the page straight
 // into the MFMA A operand; V is transposed through a wave-private LDS tile (V^T [DV][64], as in
 // the prompt kernel). Every wave keeps its own running (max, sum, accumulator) per head and map
@@ -479,14 +479,15 @@ __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
   constexpr int DT = DV / 16;
   constexpr int VBLK = DV / 32;   // (4 keys x 8 columns) blocks per lane per page
   extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
-  const int part = blockIdx.x, parts = gridDim.x, g = blockIdx.y;
+  const int grp = H / G;
+  const int n_chunk = (grp + 15) / 16;   // more than 16 heads per KV head: 16 per workgroup
+  const int part = blockIdx.x, parts = gridDim.x, g = blockIdx.y / n_chunk, c0 = (blockIdx.y % n_chunk) * 16;
   const int64_t row = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   uint16_t* v_s = sm_lds + w * (DV * KT);
   const int col = lane & 15, h = lane >> 4;
-  const int grp = H / G;
-  const int head = g * grp + (col < grp ? col : grp - 1);
+  const int head = g * grp + (c0 + col < grp ? c0 + col : grp - 1);
   const int i = pos[row];
   const int lo = window > 0 && i - window + 1 > 0 ? i - window + 1 : 0;
   const int p_lo = lo / KT, p_hi = i / KT;           // i < 0: no pages
@@ -602,7 +603,7 @@ __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
       }
     }
   }
-  if (col >= grp) return;
+  if (c0 + col >= grp) return;
   const int slot = part * 4 + w;
 #pragma unroll
   for (int m = 0; m < MAPS; ++m) {
@@ -731,7 +732,7 @@ void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
                                 const int32_t* pos, int64_t T, int H, int G, int dk, int dv, float scale, int window,
                                 int maps, float lam, float unit_eps, float out_scale, hipStream_t stream) {
   if (T == 0) return;
-  const dim3 grid((unsigned)parts, (unsigned)G, (unsigned)T);
+  const dim3 grid((unsigned)parts, (unsigned)(G * ((H / G + 15) / 16)), (unsigned)T);
   const float scale_log2 = scale * 1.4426950408889634f;
   const bool ok = maps == 2 ? launch_sm_decode_dk<2>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
                                                      scale_log2, window, dk, dv, grid, stream)
@@ -742,11 +743,10 @@ void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
                                                                                    dv, maps, lam, unit_eps, out_scale);
 }
 
-// Head sizes of the MFMA forms: dk, dv in {32, 64, 128} (one map: also 256); at most 16 heads per
-// KV head (the columns of one tile in the single-token kernel).
+// Head sizes of the MFMA forms: dk, dv in {32, 64, 128} (one map: also 256).
 bool softmax_attention_mfma_supported(int dk, int dv, int group, int maps) {
   auto ok = [&](int d) { return d == 32 || d == 64 || d == 128 || (maps == 1 && d == 256); };
-  return (maps == 1 || maps == 2) && ok(dk) && ok(dv) && group >= 1 && group <= 16;
+  return (maps == 1 || maps == 2) && ok(dk) && ok(dv) && group >= 1;
 }
 
 // prompt portions: sequence b owns rows [cu_q[b], cu_q[b + 1]) of q / gate / out, the last ones of

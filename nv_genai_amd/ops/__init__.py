@@ -555,7 +555,7 @@ def softmax_attention(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int, dk:
 
 def softmax_attention_mfma_ok(q: torch.Tensor, dk: int, dv: int, group: int = 1, maps: int = 1) -> bool:
     """The MFMA softmax attention kernels take bf16 GPU rows (16-byte aligned) with dk, dv in
-    {32, 64, 128} (one map: also 256) and at most 16 heads per KV head."""
+    {32, 64, 128} (one map: also 256)."""
     return (_gpu(q) and q.dtype == torch.bfloat16 and have_kernels() and q.stride(0) % 8 == 0
             and q.data_ptr() % 16 == 0
             and bool(kernels().softmax_attention_mfma_supported(int(dk), int(dv), int(group), int(maps))))
@@ -600,7 +600,7 @@ def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int
                                  unit_eps, out_scale, gate, out=out)
     C = kernels()
     T = q.shape[0]
-    parts = int(C.softmax_decode_parts(max(T, 1), G, int(max_ctx), int(window)))
+    parts = int(C.softmax_decode_parts(max(T, 1), G * -(-(H // G) // 16), int(max_ctx), int(window)))
     ws = torch.empty(T * H * maps * 4 * parts * (dv + 4), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
