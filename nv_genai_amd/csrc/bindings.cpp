@@ -1286,7 +1286,7 @@ void softmax_attention_prefill(Tensor out, Tensor q, c10::optional<Tensor> gate,
                                      (float)unit_eps, (float)out_scale, cur_stream(q));
 }
 
-// single-token rows on the MFMA kernel (bf16): ws is the fp32 partial workspace [T, H, maps, 4 * parts, dv + 4]
+// single-token rows on the MFMA kernel (bf16): ws is the fp32 partial workspace [T, H, maps, parts, dv + 4]
 void softmax_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c10::optional<Tensor> gate, Tensor kc,
                               Tensor vc, Tensor block_tables, Tensor tok_seq, Tensor pos, int64_t H, int64_t G,
                               int64_t dk, int64_t dv, double scale, int64_t window, int64_t maps, double lam,
@@ -1297,7 +1297,7 @@ void softmax_attention_decode(Tensor out, Tensor ws, int64_t parts, Tensor q, c1
               "softmax_attention_decode: head sizes the MFMA kernel does not take");
   TORCH_CHECK(q.stride(0) % 8 == 0 && (uintptr_t)q.data_ptr() % 16 == 0, "q rows must be 16-B aligned");
   const int64_t T = q.size(0);
-  TORCH_CHECK(parts >= 1 && parts <= 64 && ws.numel() >= T * H * maps * 4 * parts * (dv + 4) &&
+  TORCH_CHECK(parts >= 1 && parts <= 64 && ws.numel() >= T * H * maps * parts * (dv + 4) &&
               (uintptr_t)ws.data_ptr() % 16 == 0);
   TORCH_CHECK(tok_seq.numel() == T && pos.numel() == T && block_tables.dim() == 2);
   nga::launch_softmax_decode_mfma(bfp(out), ws.data_ptr<float>(), (int)parts, bfp(q), q.stride(0),

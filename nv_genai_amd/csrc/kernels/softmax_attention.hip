@@ -277,11 +277,14 @@ __global__ void __launch_bounds__(256) softmax_attention_mfma_kernel(const SmMfm
     for (int dt = 0; dt < DT; ++dt) o[m][dt] = (f32x4)(0.f);
   }
 
-  for (int t = t_first; t <= t_last; ++t) {
+  // Registers for one page in flight: with few enough of them the next page is requested before
+  // the current one is processed, so its latency hides behind the MFMA work.
+  constexpr bool PREFETCH = (MAPS * PER_K + 4 * VBLK) * 4 <= 48;
+  u16x8 kreg[MAPS][PER_K], vreg[VBLK][4];
+  auto fetch = [&](int t) {
     const int64_t blk = P.block_tables[(int64_t)b * P.max_blocks + t];
     const uint16_t* kp = P.kc + (blk * P.G + g) * (int64_t)(MAPS * KT * DK);
     const uint16_t* vp = P.vc + (blk * P.G + g) * (int64_t)(KT * DV);
-    u16x8 kreg[MAPS][PER_K], vreg[VBLK][4];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
 #pragma unroll
@@ -294,6 +297,9 @@ __global__ void __launch_bounds__(256) softmax_attention_mfma_kernel(const SmMfm
         for (int kk = 0; kk < 4; ++kk) vreg[i][kk] = load8(vp + (int64_t)(4 * (c & 15) + kk) * DV + 8 * (c >> 4));
       }
     }
+  };
+  fetch(t_first);
+  for (int t = t_first; t <= t_last; ++t) {
     __syncthreads();   // the previous page's reads are done
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
@@ -322,10 +328,12 @@ __global__ void __launch_bounds__(256) softmax_attention_mfma_kernel(const SmMfm
       }
     }
     __syncthreads();
+    if (PREFETCH && t < t_last) fetch(t + 1);
 
     const int kbase = t * KT;
     const float fd = (float)(qpos - kbase - 8 * h);
     const bool need_mask = kbase + KT - 1 > wq_lo || (W > 0 && wq_hi - kbase >= W);
+    bf16x8 pf[MAPS][2];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
       f32x4 sacc[4];
@@ -359,8 +367,8 @@ __global__ void __launch_bounds__(256) softmax_attention_mfma_kernel(const SmMfm
       const float mnew = fmaxf(mrun[m], mx);
       const float muse = mnew == -INFINITY ? 0.f : mnew;   // nothing visible yet: weights and factor 0
       const float corr = __builtin_amdgcn_exp2f(mrun[m] - muse);
+      const bool moved = mnew != mrun[m];
       mrun[m] = mnew;
-      bf16x8 pf[2];
       float ls = 0.f;
 #pragma unroll
       for (int tau = 0; tau < 4; ++tau)
@@ -368,24 +376,28 @@ __global__ void __launch_bounds__(256) softmax_attention_mfma_kernel(const SmMfm
         for (int rr = 0; rr < 4; ++rr) {
           const float pv = __builtin_amdgcn_exp2f(sacc[tau][rr] - muse);
           ls += pv;
-          pf[tau >> 1][4 * (tau & 1) + rr] = (__bf16)pv;
+          pf[m][tau >> 1][4 * (tau & 1) + rr] = (__bf16)pv;
         }
       ls += __shfl_xor(ls, 16, 64);
       ls += __shfl_xor(ls, 32, 64);
       lrun[m] = lrun[m] * corr + ls;
+      if (__ballot(moved)) {   // no maximum of this wave's rows moved: the accumulators stay as they are
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o[m][dt] *= corr;
-#pragma unroll
-      for (int gg = 0; gg < 2; ++gg) {
-        const int ch = 4 * gg + h;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const int row = 16 * dt + col;
-          const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&v_s[row * KT + ((ch ^ ((row >> 1) & 7)) * 8)]));
-          o[m][dt] = mfma16(a, pf[gg], o[m][dt]);
-        }
+        for (int dt = 0; dt < DT; ++dt) o[m][dt] *= corr;
       }
     }
+#pragma unroll
+    for (int gg = 0; gg < 2; ++gg) {
+      const int ch = 4 * gg + h;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const int row = 16 * dt + col;
+        const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&v_s[row * KT + ((ch ^ ((row >> 1) & 7)) * 8)]));
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) o[m][dt] = mfma16(a, pf[m][gg], o[m][dt]);
+      }
+    }
+    if (!PREFETCH && t < t_last) fetch(t + 1);
   }
   // lane (query col, h) holds value columns 16 dt + 4 h + rr of its query
   float inv[MAPS];
@@ -464,11 +476,12 @@ bool launch_sm_mfma_dk(const SmMfmaParams& P, int dk, int dv, dim3 grid, hipStre
 // both maps of a head: they share V). Workgroup = 4 waves = (part, KV head, token row); the row's visible pages
 // are dealt round-robin to the 4 * parts waves of the row. K fragments go from the page straight
 // into the MFMA A operand; V is transposed through a wave-private LDS tile (V^T [DV][64], as in
-// the prompt kernel). Every wave keeps its own running (max, sum, accumulator) per head and map
-// and writes them as one partial; softmax_decode_reduce merges the partials of a (row, head) in a
-// fixed order, combines the maps, normalises, gates and writes bf16.
+// the prompt kernel). Every wave keeps its own running (max, sum, accumulator) per head and map;
+// the four waves merge theirs through LDS into one partial per workgroup, and
+// softmax_decode_reduce merges the partials of a (row, head) in a fixed order, combines the maps,
+// normalises, gates and writes bf16.
 //
-// ws: fp32 [T, H, MAPS, 4 * parts, DV + 4]  (accumulator, then max (log2 domain), sum, 2 unused)
+// ws: fp32 [T, H, MAPS, parts, DV + 4]  (accumulator, then max (log2 domain), sum, 2 unused)
 template <int DK, int DV, int MAPS>
 __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
     float* __restrict__ ws, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ kc,
@@ -545,6 +558,7 @@ __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
     if (!have) continue;
     const int kbase = pg * KT;
     const bool need_mask = kbase < lo || kbase + KT - 1 > i;
+    bf16x8 pf[MAPS][2];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
       f32x4 sacc[4];
@@ -575,8 +589,8 @@ __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float mnew = fmaxf(mrun[m], mx);     // every visited page holds a visible key
       const float corr = __builtin_amdgcn_exp2f(mrun[m] - mnew);
+      const bool moved = mnew != mrun[m];
       mrun[m] = mnew;
-      bf16x8 pf[2];
       float ls = 0.f;
 #pragma unroll
       for (int tau = 0; tau < 4; ++tau)
@@ -584,35 +598,85 @@ __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
         for (int rr = 0; rr < 4; ++rr) {
           const float pv = __builtin_amdgcn_exp2f(sacc[tau][rr] - mnew);
           ls += pv;
-          pf[tau >> 1][4 * (tau & 1) + rr] = (__bf16)pv;
+          pf[m][tau >> 1][4 * (tau & 1) + rr] = (__bf16)pv;
         }
       ls += __shfl_xor(ls, 16, 64);
       ls += __shfl_xor(ls, 32, 64);
       lrun[m] = lrun[m] * corr + ls;
+      if (__ballot(moved)) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o[m][dt] *= corr;
+        for (int dt = 0; dt < DT; ++dt) o[m][dt] *= corr;
+      }
+    }
 #pragma unroll
-      for (int gg = 0; gg < 2; ++gg) {
-        const int ch = 4 * gg + h;
+    for (int gg = 0; gg < 2; ++gg) {
+      const int ch = 4 * gg + h;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const int r = 16 * dt + col;
-          const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&v_s[r * KT + ((ch ^ ((r >> 1) & 7)) * 8)]));
-          o[m][dt] = mfma16(a, pf[gg], o[m][dt]);
-        }
+      for (int dt = 0; dt < DT; ++dt) {
+        const int r = 16 * dt + col;
+        const bf16x8 a = as_bf16x8(*reinterpret_cast<const u16x8*>(&v_s[r * KT + ((ch ^ ((r >> 1) & 7)) * 8)]));
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) o[m][dt] = mfma16(a, pf[m][gg], o[m][dt]);
       }
     }
   }
-  if (c0 + col >= grp) return;
-  const int slot = part * 4 + w;
+  // merge the four waves' (max, sum, accumulator) through LDS (the V^T tiles are free now): the
+  // workgroup leaves one partial per head and map
+  __syncthreads();
+  float* ml_s = reinterpret_cast<float*>(sm_lds);          // [4][MAPS][2][16]
+  float* o_s = ml_s + 4 * MAPS * 2 * 16;                   // [MAPS][16][DV]
+  if (h == 0) {
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      ml_s[((w * MAPS + m) * 2 + 0) * 16 + col] = mrun[m];
+      ml_s[((w * MAPS + m) * 2 + 1) * 16 + col] = lrun[m];
+    }
+  }
+  __syncthreads();
+  float fac[MAPS], Mx[MAPS], Lx[MAPS];
 #pragma unroll
   for (int m = 0; m < MAPS; ++m) {
-    float* wp = ws + ((((int64_t)row * H + head) * MAPS + m) * stride + slot) * (DV + 4);
+    float M = -INFINITY;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(wp + 16 * dt + 4 * h) = o[m][dt];
-    if (h == 0) {
-      wp[DV] = mrun[m];
-      wp[DV + 1] = lrun[m];
+    for (int ww = 0; ww < 4; ++ww) M = fmaxf(M, ml_s[((ww * MAPS + m) * 2 + 0) * 16 + col]);
+    float L = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < 4; ++ww) {
+      const float mw = ml_s[((ww * MAPS + m) * 2 + 0) * 16 + col];
+      if (mw != -INFINITY) L += ml_s[((ww * MAPS + m) * 2 + 1) * 16 + col] * __builtin_amdgcn_exp2f(mw - M);
+    }
+    fac[m] = mrun[m] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mrun[m] - M);
+    Mx[m] = M;
+    Lx[m] = L;
+  }
+#pragma unroll
+  for (int ww = 0; ww < 4; ++ww) {
+    if (w == ww) {
+#pragma unroll
+      for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          f32x4* dst = reinterpret_cast<f32x4*>(o_s + (m * 16 + col) * DV + 16 * dt + 4 * h);
+          *dst = ww == 0 ? o[m][dt] * fac[m] : *dst + o[m][dt] * fac[m];
+        }
+    }
+    __syncthreads();
+  }
+  // 16 heads x DV columns per map, written by all four waves
+  const int stride_ws = parts;
+  for (int e = tid; e < MAPS * 16 * (DV / 4); e += 256) {
+    const int m = e / (16 * (DV / 4)), rem = e % (16 * (DV / 4)), cc = rem / (DV / 4), d4 = rem % (DV / 4);
+    if (c0 + cc < grp) {
+      float* wp = ws + ((((int64_t)row * H + g * grp + c0 + cc) * MAPS + m) * stride_ws + part) * (DV + 4);
+      *reinterpret_cast<f32x4*>(wp + 4 * d4) = *reinterpret_cast<const f32x4*>(o_s + (m * 16 + cc) * DV + 4 * d4);
+    }
+  }
+  if (w == 0 && h == 0 && c0 + col < grp) {
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      float* wp = ws + ((((int64_t)row * H + g * grp + c0 + col) * MAPS + m) * stride_ws + part) * (DV + 4);
+      wp[DV] = Mx[m];
+      wp[DV + 1] = Lx[m];
     }
   }
 }
@@ -628,8 +692,10 @@ __global__ void __launch_bounds__(64) softmax_decode_reduce_kernel(
   for (int m = 0; m < maps; ++m) {
     const float* wp = ws + (((int64_t)row * H + head) * maps + m) * slots * (int64_t)(dv + 4);
     float M = -INFINITY;
+#pragma unroll 4
     for (int s = 0; s < slots; ++s) M = fmaxf(M, wp[(int64_t)s * (dv + 4) + dv]);
     float L = 0.f, acc[MAXV] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
     for (int s = 0; s < slots; ++s) {
       const float* sp = wp + (int64_t)s * (dv + 4);
       const float ms = sp[dv];
@@ -663,7 +729,9 @@ template <int DK, int DV, int MAPS>
 void launch_sm_decode_one(float* ws, const uint16_t* q, int64_t q_stride, const uint16_t* kc, const uint16_t* vc,
                           const int32_t* block_tables, int max_blocks, const int32_t* tok_seq, const int32_t* pos,
                           int H, int G, float scale_log2, int window, dim3 grid, hipStream_t stream) {
-  constexpr size_t smem = (size_t)4 * DV * 64 * sizeof(uint16_t);
+  constexpr size_t tiles = (size_t)4 * DV * 64 * sizeof(uint16_t);
+  constexpr size_t merge = (size_t)(4 * MAPS * 2 * 16 + MAPS * 16 * DV) * sizeof(float);
+  constexpr size_t smem = tiles > merge ? tiles : merge;
   static bool attr_set = false;
   if (smem > 65536 && !attr_set) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&softmax_decode_mfma_kernel<DK, DV, MAPS>),
@@ -725,7 +793,7 @@ int softmax_decode_parts(int rows, int G, int max_ctx, int window) {
   return p < 1 ? 1 : (p > 32 ? 32 : p);
 }
 
-// ws: fp32 [T, H, maps, 4 * parts, dv + 4]
+// ws: fp32 [T, H, maps, parts, dv + 4]
 void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint16_t* q, int64_t q_stride,
                                 const uint16_t* gate, int64_t g_stride, const uint16_t* kc, const uint16_t* vc,
                                 const int32_t* block_tables, int max_blocks, const int32_t* tok_seq,
@@ -739,7 +807,7 @@ void launch_softmax_decode_mfma(uint16_t* out, float* ws, int parts, const uint1
                             : launch_sm_decode_dk<1>(ws, q, q_stride, kc, vc, block_tables, max_blocks, tok_seq, pos, H, G,
                                                      scale_log2, window, dk, dv, grid, stream);
   if (!ok) abort();   // the caller checks softmax_attention_mfma_supported
-  softmax_decode_reduce_kernel<<<dim3((unsigned)T, (unsigned)H), 64, 0, stream>>>(out, ws, 4 * parts, gate, g_stride, H,
+  softmax_decode_reduce_kernel<<<dim3((unsigned)T, (unsigned)H), 64, 0, stream>>>(out, ws, parts, gate, g_stride, H,
                                                                                    dv, maps, lam, unit_eps, out_scale);
 }
 

@@ -601,7 +601,7 @@ def softmax_attention_rows(q, kc, vc, block_tables, tok_seq, pos, H: int, G: int
     C = kernels()
     T = q.shape[0]
     parts = int(C.softmax_decode_parts(max(T, 1), G * -(-(H // G) // 16), int(max_ctx), int(window)))
-    ws = torch.empty(T * H * maps * 4 * parts * (dv + 4), dtype=torch.float32, device=q.device)
+    ws = torch.empty(T * H * maps * parts * (dv + 4), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
     C.softmax_attention_decode(out, ws, parts, q, gate, kc, vc, block_tables, tok_seq, pos, H, G, dk, dv,
