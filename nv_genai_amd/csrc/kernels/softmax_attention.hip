@@ -535,21 +535,26 @@ __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
     const uint16_t* vp = vc + (blk * G + g) * (int64_t)(KT * DV);
     __syncthreads();   // the previous page's reads of this wave's tile are done
     if (have) {
+      // all of the page's V loads in flight together, then the transposed stores
+      u16x8 vreg[VBLK][4];
 #pragma unroll
       for (int bi = 0; bi < VBLK; ++bi) {
         const int c = lane + 64 * bi;            // block: keys 4 * (c & 15) .. + 3, columns 8 * (c >> 4) .. + 7
-        const int kb = c & 15, dc = c >> 4;
-        u16x8 vreg[4];
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) vreg[kk] = load8(vp + (int64_t)(4 * kb + kk) * DV + 8 * dc);
+        for (int kk = 0; kk < 4; ++kk) vreg[bi][kk] = load8(vp + (int64_t)(4 * (c & 15) + kk) * DV + 8 * (c >> 4));
+      }
+#pragma unroll
+      for (int bi = 0; bi < VBLK; ++bi) {
+        const int c = lane + 64 * bi;
+        const int kb = c & 15, dc = c >> 4;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int r = 8 * dc + e;
           u16x4 tv;
-          tv[0] = vreg[0][e];
-          tv[1] = vreg[1][e];
-          tv[2] = vreg[2][e];
-          tv[3] = vreg[3][e];
+          tv[0] = vreg[bi][0][e];
+          tv[1] = vreg[bi][1][e];
+          tv[2] = vreg[bi][2][e];
+          tv[3] = vreg[bi][3][e];
           *reinterpret_cast<u16x4*>(&v_s[r * KT + (((kb >> 1) ^ ((r >> 1) & 7)) * 8) + 4 * (kb & 1)]) = tv;
         }
       }
@@ -561,16 +566,20 @@ __global__ void __launch_bounds__(256) softmax_decode_mfma_kernel(
     bf16x8 pf[MAPS][2];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
-      f32x4 sacc[4];
+      // the map's K fragments of the whole page in flight together (one round trip), then the MFMAs
+      u16x8 kf[4][DS];
 #pragma unroll
       for (int tau = 0; tau < 4; ++tau) {
         const int kr = 32 * (tau >> 1) + 8 * (col >> 2) + 4 * (tau & 1) + (col & 3);
+#pragma unroll
+        for (int s2 = 0; s2 < DS; ++s2) kf[tau][s2] = load8(kp + m * KT * DK + kr * DK + 32 * s2 + 8 * h);
+      }
+      f32x4 sacc[4];
+#pragma unroll
+      for (int tau = 0; tau < 4; ++tau) {
         sacc[tau] = (f32x4)(0.f);
 #pragma unroll
-        for (int s2 = 0; s2 < DS; ++s2) {
-          const bf16x8 a = as_bf16x8(load8(kp + m * KT * DK + kr * DK + 32 * s2 + 8 * h));
-          sacc[tau] = mfma16(a, qf[m][s2], sacc[tau]);
-        }
+        for (int s2 = 0; s2 < DS; ++s2) sacc[tau] = mfma16(as_bf16x8(kf[tau][s2]), qf[m][s2], sacc[tau]);
       }
       float mx = -INFINITY;
 #pragma unroll
