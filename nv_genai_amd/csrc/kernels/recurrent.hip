@@ -23,6 +23,12 @@ template <typename T> __device__ __forceinline__ float ldf(const T* p);
 template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf2f(*p); }
 template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
 
+// 1 / (1 + 2^(-z log2 e)) on the hardware exp2 and reciprocal (1 ulp each): the activations are
+// recomputed by every value tile of a head, so their cost is on the scan's critical path
+__device__ __forceinline__ float sigmoid_fast(float z) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+}
+
 constexpr int TC = 16;   // rows staged per pass
 
 // proj row: [q_pre (H*d) | f_pre (H*d) | v (H*dv) | ...]. cu == nullptr: segment b is row b.
@@ -85,8 +91,8 @@ __global__ void __launch_bounds__(256) hgrn2_scan_kernel(float* __restrict__ out
       const int e = tid + 256 * x, i = e % DP;
       if (i < d) {
         const float lw = lower[qoff + i];
-        qs[e] = rq[x] / (1.0f + expf(-rq[x]));
-        fs[e] = lw + (1.0f - lw) * (1.0f / (1.0f + expf(-(rf[x] + f_bias[qoff + i]))));
+        qs[e] = rq[x] * sigmoid_fast(rq[x]);
+        fs[e] = lw + (1.0f - lw) * sigmoid_fast(rf[x] + f_bias[qoff + i]);
       } else {
         qs[e] = 0.f;
         fs[e] = 1.f;
@@ -99,7 +105,7 @@ __global__ void __launch_bounds__(256) hgrn2_scan_kernel(float* __restrict__ out
     }
     __syncthreads();
     if (tc + TC < t1) fetch(tc + TC);   // lands while this pass computes
-    for (int tt = 0; tt < nt; ++tt) {
+    auto row = [&](int tt) {
       const float vv = vs[tt * VT + j];
       const float4* fr = reinterpret_cast<const float4*>(fs + tt * DP + rg * NR);
       const float4* qr = reinterpret_cast<const float4*>(qs + tt * DP + rg * NR);
@@ -116,6 +122,12 @@ __global__ void __launch_bounds__(256) hgrn2_scan_kernel(float* __restrict__ out
         }
       }
       part[tt * 256 + tid] = p;
+    };
+    if (nt == TC) {   // full pass: unrolled, so the LDS reads of later rows run ahead of the recurrence
+#pragma unroll
+      for (int tt = 0; tt < TC; ++tt) row(tt);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) row(tt);
     }
     __syncthreads();
     for (int e = tid; e < nt * VT; e += 256) {
