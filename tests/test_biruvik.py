@@ -52,9 +52,9 @@ def cfg_odd():
 
 def cfg_tiles():
     """Head sizes the MFMA kernels take (multiples of 32), unequal per layer."""
-    return cfg_dict([attn(heads=4, kv_heads=2, dim=32, vdim=64, scale=0.18), latent(heads=3, dim=32, vdim=32, kv_rank=64),
+    return cfg_dict([attn(heads=4, kv_heads=2, dim=64, vdim=32, scale=0.12), latent(heads=3, dim=16, vdim=32, kv_rank=64),
                      hgrn(heads=2, dim=32, vdim=64),
-                     attn(heads=2, kv_heads=1, dim=64, vdim=32, scale=0.12, every=64, ff=None),
+                     attn(heads=2, kv_heads=1, dim=32, vdim=128, scale=0.18, every=64, ff=None),
                      latent(heads=18, dim=16, vdim=16, kv_rank=128, window=130, scale=0.2)], width=48)
 
 
