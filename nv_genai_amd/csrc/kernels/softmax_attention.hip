@@ -240,7 +240,8 @@ softmax_attention_mfma_kernel(const SmMfmaParams P) {
   extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
   uint16_t* k_s = sm_lds;                       // [MAPS][KT * DK]
   uint16_t* v_s = sm_lds + MAPS * KT * DK;      // [DV * KT]
-  const int tile = blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
+  // the last row blocks of a sequence see the most pages: they are launched first
+  const int tile = gridDim.x - 1 - blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
   const int q0 = P.cu_q[b], qlen = P.cu_q[b + 1] - q0;
   if (tile * 64 >= qlen) return;
   const int ctx = P.ctx_lens[b];
