@@ -8,7 +8,11 @@
 //                      place, k and v into the token's page slot
 //   softmax_attention  one wave per (token row, head), prompt portions and single-token rows
 //                      alike: keys by lane for q.k, value columns by lane for w.V, running
-//                      maximum and sum per map (fp32)
+//                      maximum and sum per map (fp32); any sizes, bf16 and fp32
+//   softmax_attention_mfma (bf16)  one workgroup per (64-row block of a sequence, head): MFMA q.k
+//                      and p.V tiles over the pages the block can see, both maps in one wave
+//   softmax_decode_mfma + softmax_decode_reduce (bf16)  single-token rows: the heads of a KV head
+//                      are the tile columns, a row's pages are dealt to several workgroups
 //
 // Pages: K [blocks, G * maps, 64, dk], V [blocks, G, 64, dv] (T = bf16 or fp32). A head has
 // `maps` score maps (1 or 2) that share its values: q head (h, m) is column block h * maps + m,
