@@ -597,3 +597,47 @@ def test_mfma_forms_run_and_agree_with_the_row_kernel():
         got1 = ops.softmax_attention_rows(q[pick].contiguous(), kc, vc, bts, seq[pick].contiguous(),
                                           pos[pick].contiguous(), H, G, dk, dv, dk ** -0.5, max_ctx=1536, **kw).float()
         assert (got1 - want[pick]).abs().max().item() < 0.03 * max(1.0, want.abs().max().item()), ("single-token kernel", H, G, dk, dv, W)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_trace_runner_replays_a_schedule(device, tmp_path, monkeypatch, capsys):
+    """The trace runner on a model folder: steps as JSON lines on standard input (a prompt in two
+    portions, a second request beside single tokens of the first, requests ended and their names
+    used again), logits files of the wanted places, a ``done`` line per step."""
+    import io
+
+    import numpy as np
+
+    from nv_genai_amd.tools import trace_run
+    from nv_genai_amd.utils.checkpoint import save_weights
+
+    cd = cfg_dict([attn(), latent(window=9), hgrn()])
+    cfg = BiruvikConfig.from_dict(cd)
+    w = random_weights(cfg, 8, torch.bfloat16)
+    model_dir, out_dir = tmp_path / "model", tmp_path / "out"
+    save_weights(w, str(model_dir))
+    (model_dir / "config.json").write_text(json.dumps(cd))
+    a, b = tokens(80, seed=51), tokens(30, seed=52)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:65], "want": [0, 64]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[65:78], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[:29], "want": [28]}, {"id": "a", "tokens": a[78:79], "want": [0]}],
+              "end": []},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[79:], "want": [0]}, {"id": "b", "tokens": b[29:], "want": [0]}],
+              "end": ["a", "b"]},
+             {"step": 4, "entries": [{"id": "a", "tokens": b[:5], "want": [4]}], "end": ["a"]}]
+    monkeypatch.setattr("sys.stdin", io.StringIO("".join(json.dumps(s) + "\n" for s in steps)))
+    rc = trace_run.main(["--model", str(model_dir), "--dtype", "float32", "--out", str(out_dir), "--max-tokens", "192",
+                         "--device", device])
+    assert rc == 0
+    assert [l for l in capsys.readouterr().out.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    wa, wb = O.forward(cd, w, a), O.forward(cd, w, b)
+    V = cd["vocab"]
+
+    def rows(i):
+        return torch.from_numpy(np.fromfile(out_dir / f"{i}.f32", dtype="<f4").reshape(-1, V).copy())
+
+    assert not (out_dir / "1.f32").exists()
+    close(rows(0), wa[[0, 64]], "float32", "first portion")
+    close(rows(2), torch.stack([wb[28], wa[78]]), "float32", "a portion beside a single token")
+    close(rows(3), torch.stack([wa[79], wb[29]]), "float32", "last tokens")
+    close(rows(4), wb[4:5], "float32", "a name used again")
